@@ -162,3 +162,168 @@ class Qwen2Config:
         return (
             2 * self.num_hidden_layers * self.num_key_value_heads * self.head_dim * elem_bytes
         )
+
+
+@dataclass(frozen=True)
+class LatentMixerConfig:
+    """Sizes and constants of one latent-attention mixer (``layers[i].mixer``)."""
+
+    heads: int
+    dim: int          # unrotated query/key dims per head
+    rot_dim: int      # rotated query/key dims per head (the key's are shared by the heads)
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    rot_base: float
+    rot_dims: int     # how many of the rotated part's dims turn
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "LatentMixerConfig":
+        need = lambda key: _require_in(raw, key, where)
+        rot = raw.get("rot") or {}
+        rot_dim = int(need("rot_dim"))
+        dim = int(need("dim"))
+        cfg = cls(
+            heads=int(need("heads")), dim=dim, rot_dim=rot_dim, vdim=int(need("vdim")),
+            q_rank=int(need("q_rank")), kv_rank=int(need("kv_rank")),
+            scale=float(raw["scale"]) if raw.get("scale") is not None else (dim + rot_dim) ** -0.5,
+            rot_base=float(rot.get("base", 10000.0)),
+            rot_dims=int(rot.get("dims", rot_dim)),
+        )
+        for name in ("heads", "dim", "vdim", "q_rank", "kv_rank"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if cfg.rot_dim < 0 or cfg.rot_dims < 0 or cfg.rot_dims > cfg.rot_dim or cfg.rot_dims % 2:
+            raise ConfigError(f"{where}: {cfg.rot_dims} rotated dims (even) of a rotated part of {cfg.rot_dim}")
+        if cfg.rot_dims and not cfg.rot_base > 0:
+            raise ConfigError(f"{where}.rot.base must be positive")
+        return cfg
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim,
+                "q_rank": self.q_rank, "kv_rank": self.kv_rank, "scale": self.scale,
+                "rot": {"base": self.rot_base, "dims": self.rot_dims}}
+
+
+@dataclass(frozen=True)
+class FeedForwardConfig:
+    """``layers[i].mlp``: a dense gated feed-forward (`experts` 0) or routed experts."""
+
+    ff: int
+    limit: float
+    experts: int = 0
+    top: int = 0
+    router_scale: float = 1.0
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "FeedForwardConfig":
+        kind = _require_in(raw, "kind", where)
+        if kind == "dense":
+            cfg = cls(ff=int(_require_in(raw, "ff", where)), limit=float(_require_in(raw, "limit", where)))
+        elif kind == "moe":
+            expert = _require_in(raw, "expert", where)
+            router = _require_in(raw, "router", where)
+            cfg = cls(ff=int(_require_in(expert, "ff", where + ".expert")),
+                      limit=float(_require_in(expert, "limit", where + ".expert")),
+                      experts=int(_require_in(router, "experts", where + ".router")),
+                      top=int(_require_in(router, "top", where + ".router")),
+                      router_scale=float(router.get("scale", 1.0)))
+            if not 0 < cfg.top <= cfg.experts:
+                raise ConfigError(f"{where}: top {cfg.top} of {cfg.experts} experts")
+        else:
+            raise ConfigError(f"{where}.kind {kind!r} is not implemented; known: dense, moe")
+        if cfg.ff <= 0 or not cfg.limit > 0:
+            raise ConfigError(f"{where}: ff and limit must be positive")
+        return cfg
+
+    def to_dict(self) -> dict:
+        if not self.experts:
+            return {"kind": "dense", "ff": self.ff, "limit": self.limit}
+        return {"kind": "moe", "expert": {"ff": self.ff, "limit": self.limit},
+                "router": {"experts": self.experts, "top": self.top, "scale": self.router_scale}}
+
+
+@dataclass(frozen=True)
+class TalolornLayerConfig:
+    mixer: LatentMixerConfig
+    mlp: FeedForwardConfig | None
+    weights_of: int | None = None     # the layer whose tensors this one uses
+
+
+def _require_in(raw: dict, key: str, where: str):
+    if not isinstance(raw, dict) or key not in raw:
+        raise ConfigError(f"config.json has no {where}.{key}")
+    return raw[key]
+
+
+@dataclass(frozen=True)
+class TalolornConfig:
+    """The Talolorn decoder: a scaled embedding; layers of one RMS norm whose output a
+    latent-attention mixer and a feed-forward (dense or routed experts, or none) both read,
+    their sum entering the residual stream times ``residual_mult``; a final RMS norm and an
+    untied head.  ``layers`` lists the layers in order; one with ``weights_of: j`` runs layer
+    j's tensors over a cache of its own."""
+
+    vocab: int
+    width: int
+    embedding_scale: float
+    norm_eps: float
+    residual_mult: float
+    layers: tuple
+    architecture: str = "Talolorn"
+    eos_token_ids: tuple = ()
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "TalolornConfig":
+        entries = _require(raw, "layers")
+        if not isinstance(entries, list) or not entries:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(entries):
+            where = f"layers[{i}]"
+            kind = _require_in(entry, "type", where)
+            if kind != "latent_attention":
+                raise ConfigError(f"{where}.type {kind!r} is not implemented; known: latent_attention")
+            mlp = entry.get("mlp")
+            shared = entry.get("weights_of")
+            layers.append(TalolornLayerConfig(
+                mixer=LatentMixerConfig.from_dict(_require_in(entry, "mixer", where), where + ".mixer"),
+                mlp=None if mlp is None else FeedForwardConfig.from_dict(mlp, where + ".mlp"),
+                weights_of=None if shared is None else int(shared)))
+        cfg = cls(
+            vocab=int(_require(raw, "vocab")), width=int(_require(raw, "width")),
+            embedding_scale=float((raw.get("embedding") or {}).get("scale", 1.0)),
+            norm_eps=float(_require_in(_require(raw, "norm"), "eps", "norm")),
+            residual_mult=float(raw.get("residual_mult", 1.0)),
+            layers=tuple(layers),
+            architecture=str(raw.get("architecture") or (raw.get("architectures") or ["Talolorn"])[0]),
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("vocab and width must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        for i, layer in enumerate(self.layers):
+            j = layer.weights_of
+            if j is None:
+                continue
+            if not 0 <= j < len(self.layers) or self.layers[j].weights_of is not None:
+                raise ConfigError(f"layers[{i}].weights_of names {j}, which is no layer with tensors of its own")
+            if (self.layers[j].mixer, self.layers[j].mlp) != (layer.mixer, layer.mlp):
+                raise ConfigError(f"layers[{i}] uses the tensors of layer {j} but differs from it")
+
+    def to_dict(self) -> dict:
+        layers = []
+        for layer in self.layers:
+            entry = {"type": "latent_attention", "mixer": layer.mixer.to_dict(),
+                     "mlp": None if layer.mlp is None else layer.mlp.to_dict()}
+            if layer.weights_of is not None:
+                entry["weights_of"] = layer.weights_of
+            layers.append(entry)
+        return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
+                "embedding": {"scale": self.embedding_scale}, "norm": {"eps": self.norm_eps},
+                "residual_mult": self.residual_mult, "layers": layers}

@@ -34,9 +34,14 @@ def _load_builtin() -> None:
 
 def architecture_of(raw: dict) -> str:
     names = raw.get("architectures")
-    if not names:
-        raise ConfigError("config.json has no 'architectures' entry naming the model class")
-    return names[0]
+    if names:
+        return names[0]
+    # some families name their one class in a string of its own
+    name = raw.get("architecture")
+    if isinstance(name, str) and name:
+        return name
+    raise ConfigError("config.json has no 'architectures' (or 'architecture') entry naming the "
+                      "model class")
 
 
 def resolve(raw: dict):

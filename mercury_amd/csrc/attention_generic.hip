@@ -17,15 +17,17 @@
 #include "mercury_kernels.h"
 
 #define AG_MAX_D 256
+#define AG_MAX_WIDE 1024   // keys and values of unequal widths (one shared latent per token)
 
-template <typename T>
+template <typename T, int MAXD>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int table_stride, int page_shift, int n_q, int n_kv,
-    int d, float scale, int window, float score_cap, const float* __restrict__ distance_slopes) {
-  __shared__ float qs[AG_MAX_D];
+    int d, int dv, float scale, int window, float score_cap,
+    const float* __restrict__ distance_slopes) {
+  __shared__ float qs[MAXD];
   __shared__ float probs[MK_WAVE];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int kvh = head / (n_q / n_kv);
@@ -40,9 +42,9 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   __syncthreads();
 
   float m = -INFINITY, l = 0.f;
-  float acc[AG_MAX_D / MK_WAVE];
+  float acc[MAXD / MK_WAVE];
 #pragma unroll
-  for (int c = 0; c < AG_MAX_D / MK_WAVE; ++c) acc[c] = 0.f;
+  for (int c = 0; c < MAXD / MK_WAVE; ++c) acc[c] = 0.f;
 
   for (int j0 = first; j0 <= pos; j0 += MK_WAVE) {
     const int j = j0 + lane;
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const float corr = expf(m - m_new);  // 0 on the first chunk, where m is -inf
     l = l * corr + wave_sum(p);
 #pragma unroll
-    for (int c = 0; c < AG_MAX_D / MK_WAVE; ++c) acc[c] *= corr;
+    for (int c = 0; c < MAXD / MK_WAVE; ++c) acc[c] *= corr;
     __syncthreads();
     probs[lane] = p;
     __syncthreads();
@@ -74,12 +76,12 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
       const int page = table[key >> page_shift];
       // values are stored transposed within a page: [page, kv head, dim, slot]
       const T* vcol =
-          v_cache + ((size_t)page * n_kv + kvh) * page_size * d + (key & page_mask);
+          v_cache + ((size_t)page * n_kv + kvh) * page_size * dv + (key & page_mask);
       const float pj = probs[jj];
 #pragma unroll
-      for (int c = 0; c < AG_MAX_D / MK_WAVE; ++c) {
+      for (int c = 0; c < MAXD / MK_WAVE; ++c) {
         const int dim = lane + c * MK_WAVE;
-        if (dim < d)
+        if (dim < dv)
           acc[c] = fmaf(pj, Elem<T>::load(vcol + (size_t)dim * page_size), acc[c]);
       }
     }
@@ -88,10 +90,48 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
 
   const float inv = 1.f / l;
 #pragma unroll
-  for (int c = 0; c < AG_MAX_D / MK_WAVE; ++c) {
+  for (int c = 0; c < MAXD / MK_WAVE; ++c) {
     const int dim = lane + c * MK_WAVE;
-    if (dim < d) Elem<T>::store(out + (size_t)t * out_stride + head * d + dim, acc[c] * inv);
+    if (dim < dv) Elem<T>::store(out + (size_t)t * out_stride + head * dv + dim, acc[c] * inv);
   }
+}
+
+// Keys of width d and values of width dv (values transposed within a page: [page, kv head, dv,
+// slot]); d == dv is the ordinary case.
+extern "C" int mk_attention_generic_kv(const void* q, int q_stride, void* out, int out_stride,
+                                       const void* k_cache, const void* v_cache, int dtype,
+                                       const int* positions, const int* token_seq,
+                                       const int* block_table, int table_stride, int page_size,
+                                       int n_q, int n_kv, int d, int dv, float scale, int window,
+                                       float score_cap, const float* distance_slopes, int tokens,
+                                       hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv > 0 && d > 0 && dv > 0, "attention: bad sizes");
+  MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
+             n_q, n_kv);
+  const int widest = d > dv ? d : dv;
+  MK_REQUIRE(widest <= AG_MAX_WIDE, "attention: head size %d exceeds the supported maximum %d",
+             widest, AG_MAX_WIDE);
+  MK_REQUIRE(mk_is_pow2(page_size), "attention: page size %d is not a power of two", page_size);
+  MK_REQUIRE(n_q <= 65535, "attention: too many heads (%d)", n_q);
+  MK_REQUIRE(window >= 0, "attention: negative window");
+  MK_REQUIRE(score_cap >= 0.f, "attention: negative score cap");
+  if (tokens == 0) return 0;
+  dim3 grid(tokens, n_q);
+#define AG_LAUNCH(T, MAXD)                                                                      \
+  attention_generic_kernel<T, MAXD><<<grid, MK_WAVE, 0, stream>>>(                              \
+      (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_cache, (const T*)v_cache,         \
+      positions, token_seq, block_table, table_stride, mk_log2(page_size), n_q, n_kv, d, dv,    \
+      scale, window, score_cap, distance_slopes)
+  if (dtype == MK_F32) {
+    if (widest <= AG_MAX_D) AG_LAUNCH(float, AG_MAX_D); else AG_LAUNCH(float, AG_MAX_WIDE);
+  } else if (dtype == MK_BF16) {
+    if (widest <= AG_MAX_D) AG_LAUNCH(bf16_t, AG_MAX_D); else AG_LAUNCH(bf16_t, AG_MAX_WIDE);
+  } else {
+    MK_REQUIRE(false, "attention: unknown dtype %d", dtype);
+  }
+#undef AG_LAUNCH
+  MK_LAUNCH_CHECK("attention_generic");
+  return 0;
 }
 
 extern "C" int mk_attention_generic(const void* q, int q_stride, void* out, int out_stride,
@@ -101,29 +141,9 @@ extern "C" int mk_attention_generic(const void* q, int q_stride, void* out, int 
                                     int n_q, int n_kv, int d, float scale, int window,
                                     float score_cap, const float* distance_slopes, int tokens,
                                     hipStream_t stream) {
-  MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv > 0 && d > 0, "attention: bad sizes");
-  MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
-             n_q, n_kv);
   MK_REQUIRE(d <= AG_MAX_D, "attention: head size %d exceeds the supported maximum %d", d,
              AG_MAX_D);
-  MK_REQUIRE(mk_is_pow2(page_size), "attention: page size %d is not a power of two", page_size);
-  MK_REQUIRE(n_q <= 65535, "attention: too many heads (%d)", n_q);
-  MK_REQUIRE(window >= 0, "attention: negative window");
-  MK_REQUIRE(score_cap >= 0.f, "attention: negative score cap");
-  if (tokens == 0) return 0;
-  dim3 grid(tokens, n_q);
-  if (dtype == MK_F32)
-    attention_generic_kernel<float><<<grid, MK_WAVE, 0, stream>>>(
-        (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_cache,
-        (const float*)v_cache, positions, token_seq, block_table, table_stride,
-        mk_log2(page_size), n_q, n_kv, d, scale, window, score_cap, distance_slopes);
-  else if (dtype == MK_BF16)
-    attention_generic_kernel<bf16_t><<<grid, MK_WAVE, 0, stream>>>(
-        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_cache,
-        (const bf16_t*)v_cache, positions, token_seq, block_table, table_stride,
-        mk_log2(page_size), n_q, n_kv, d, scale, window, score_cap, distance_slopes);
-  else
-    MK_REQUIRE(false, "attention: unknown dtype %d", dtype);
-  MK_LAUNCH_CHECK("attention_generic");
-  return 0;
+  return mk_attention_generic_kv(q, q_stride, out, out_stride, k_cache, v_cache, dtype, positions,
+                                 token_seq, block_table, table_stride, page_size, n_q, n_kv, d, d,
+                                 scale, window, score_cap, distance_slopes, tokens, stream);
 }

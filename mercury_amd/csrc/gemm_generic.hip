@@ -15,7 +15,14 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
                                                            const T* __restrict__ w,
                                                            const TB* __restrict__ bias,
                                                            TO* __restrict__ out, int M, int N,
-                                                           int K, int lda, int ldo) {
+                                                           int K, int lda, int ldo,
+                                                           long long x_batch, long long w_batch,
+                                                           long long o_batch) {
+  // blockIdx.z: one of several independent products (a head's own matrix over the head's own
+  // columns of x), each at its own offset into x, w and out
+  x += (size_t)blockIdx.z * x_batch;
+  w += (size_t)blockIdx.z * w_batch;
+  out += (size_t)blockIdx.z * o_batch;
   __shared__ float xs[GK][GT + 4];
   __shared__ float ws[GK][GT + 4];
   const int tid = threadIdx.x;
@@ -81,14 +88,17 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 template <typename T, typename TO, int ACC>
 static void launch_generic(const void* x, const void* w, const void* bias, int bias_dtype,
                            void* out, int M, int N, int K, int lda, int ldo,
-                           hipStream_t stream) {
-  dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT);
+                           hipStream_t stream, int batch = 1, long long x_batch = 0,
+                           long long w_batch = 0, long long o_batch = 0) {
+  dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT, batch);
   if (bias && bias_dtype == MK_BF16)
     gemm_generic_kernel<T, TO, ACC, bf16_t><<<grid, 256, 0, stream>>>(
-        (const T*)x, (const T*)w, (const bf16_t*)bias, (TO*)out, M, N, K, lda, ldo);
+        (const T*)x, (const T*)w, (const bf16_t*)bias, (TO*)out, M, N, K, lda, ldo, x_batch,
+        w_batch, o_batch);
   else
     gemm_generic_kernel<T, TO, ACC, float><<<grid, 256, 0, stream>>>(
-        (const T*)x, (const T*)w, (const float*)bias, (TO*)out, M, N, K, lda, ldo);
+        (const T*)x, (const T*)w, (const float*)bias, (TO*)out, M, N, K, lda, ldo, x_batch,
+        w_batch, o_batch);
 }
 
 extern "C" int mk_linear_generic(const void* x, const void* w, int dtype, const void* bias,
@@ -117,5 +127,33 @@ extern "C" int mk_linear_generic(const void* x, const void* w, int dtype, const 
     MK_REQUIRE(false, "linear: unsupported dtypes in=%d out=%d", dtype, out_dtype);
   }
   MK_LAUNCH_CHECK("linear_generic");
+  return 0;
+}
+
+// `batch` independent products in one launch: product b reads x + b * x_batch (rows lda apart),
+// w + b * w_batch ([N, K]) and writes out + b * o_batch (rows ldo apart), all in elements.
+// What a mixer with a matrix of its own per head needs: x[t, head, :] W[head]^T.
+extern "C" int mk_linear_batched_generic(const void* x, const void* w, int dtype, void* out,
+                                         int out_dtype, int M, int N, int K, int lda, int ldo,
+                                         int batch, long long x_batch, long long w_batch,
+                                         long long o_batch, hipStream_t stream) {
+  MK_REQUIRE(M >= 0 && N > 0 && K > 0 && batch > 0, "batched linear: bad sizes M=%d N=%d K=%d B=%d",
+             M, N, K, batch);
+  MK_REQUIRE(lda >= K && ldo >= N, "batched linear: leading dimensions %d/%d smaller than K=%d/N=%d",
+             lda, ldo, K, N);
+  MK_REQUIRE((M + GT - 1) / GT <= 65535 && batch <= 65535, "batched linear: too large for one launch");
+  if (M == 0) return 0;
+  if (dtype == MK_F32 && out_dtype == MK_F32)
+    launch_generic<float, float, 0>(x, w, nullptr, MK_F32, out, M, N, K, lda, ldo, stream, batch,
+                                    x_batch, w_batch, o_batch);
+  else if (dtype == MK_BF16 && out_dtype == MK_F32)
+    launch_generic<bf16_t, float, 0>(x, w, nullptr, MK_F32, out, M, N, K, lda, ldo, stream, batch,
+                                     x_batch, w_batch, o_batch);
+  else if (dtype == MK_BF16 && out_dtype == MK_BF16)
+    launch_generic<bf16_t, bf16_t, 0>(x, w, nullptr, MK_F32, out, M, N, K, lda, ldo, stream, batch,
+                                      x_batch, w_batch, o_batch);
+  else
+    MK_REQUIRE(false, "batched linear: unsupported dtypes in=%d out=%d", dtype, out_dtype);
+  MK_LAUNCH_CHECK("linear_batched_generic");
   return 0;
 }

@@ -10,7 +10,11 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 21
+#define MK_ABI_VERSION 22
+
+// Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
+// g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
+enum { MK_ACT_SILU = 0, MK_ACT_SWISH_CLAMP = 1 };
 
 #ifdef __cplusplus
 extern "C" {
@@ -103,6 +107,70 @@ int mk_qkv_finish(const float* partials, int num_partials, long long partial_str
 // numbers wherever they are drawn.
 int mk_fill_normal(void* out, int dtype, long long n, unsigned long long key, float mean,
                    float std, hipStream_t stream);
+
+// mk_attention_generic with keys of width d and values of width dv (the value cache is
+// [pages, n_kv, dv, page_size]); the output rows hold n_q heads of dv.
+int mk_attention_generic_kv(const void* q, int q_stride, void* out, int out_stride,
+                            const void* k_cache, const void* v_cache, int dtype,
+                            const int* positions, const int* token_seq, const int* block_table,
+                            int table_stride, int page_size, int n_q, int n_kv, int d, int dv,
+                            float scale, int window, float score_cap,
+                            const float* distance_slopes, int tokens, hipStream_t stream);
+
+// `batch` independent products y_b = x_b W_b^T in one launch: x_b = x + b * x_batch (rows lda
+// apart), W_b = w + b * w_batch ([N, K]), y_b = out + b * o_batch (rows ldo apart); offsets in
+// elements.  A matrix of its own per head over the head's own columns of x.
+int mk_linear_batched_generic(const void* x, const void* w, int dtype, void* out, int out_dtype,
+                              int M, int N, int K, int lda, int ldo, int batch, long long x_batch,
+                              long long w_batch, long long o_batch, hipStream_t stream);
+
+// Attention through a shared latent, the per-token side.  down [T, down_stride] (float32)
+// holds a token's [query latent (q_rank) | key/value latent (kv_rank) | rotated key part
+// (rot)].  The query latent is RMS-normed (q_norm_w) into q_latent [T, q_rank]; the key/value
+// latent is RMS-normed (kv_norm_w) and, with the rotated part turned by the token's position
+// (the first rot_dims dims of it, pairs (2i, 2i + 1) when interleaved, else (i, i + rot_dims /
+// 2); angle tables [positions, rot_dims / 2]), written to the paged cache as one key row
+// [kv_rank + rot] of one shared head, the normed latent once more as that head's value,
+// transposed within the page ([pages, kv_rank, page_size]).  q_rank = 0: no query latent.
+int mk_latent_prepare(const float* down, int down_stride, int q_rank, int kv_rank, int rot,
+                      const void* q_norm_w, const void* kv_norm_w, int norm_dtype, float eps,
+                      const float* cos_table, const float* sin_table, int table_positions,
+                      int rot_dims, int interleaved, const int* positions, const int* token_seq,
+                      const int* block_table, int table_stride, void* q_latent, void* k_cache,
+                      void* v_cache, int dtype, int page_size, int write_kv, int tokens,
+                      hipStream_t stream);
+
+// q [T, heads, dim + rot] -> out[t, head, out_offset .. out_offset + rot) of rows
+// [heads, out_width]: every head's rotated part, turned by the token's position.
+int mk_latent_query_tail(const void* q, int dtype, int heads, int dim, int rot,
+                         const float* cos_table, const float* sin_table, int table_positions,
+                         int rot_dims, int interleaved, const int* positions, void* out,
+                         int out_width, int out_offset, int tokens, hipStream_t stream);
+
+// Routing: scores = softmax(logits [T, experts], float32); ids / weights [T, top]: the `top`
+// largest scores' experts (ties: the lower index) and score * scale, the scores divided by
+// the chosen ones' sum first when `renormalize`.
+int mk_route_topk(const float* logits, int experts, int top, float scale, int renormalize,
+                  int* ids, float* weights, int tokens, hipStream_t stream);
+
+// Experts token by token: act [T * top, ff] = gate_act(Wg[e] x_t, Wu[e] x_t) for
+// w [experts, 2 ff, K] = [gate | up]; then y [T, N] (float32) += sum_j weights[t, j] *
+// Wd[e_j] act[(t, j)] for w [experts, N, ff], j ascending.
+int mk_expert_gated(const void* x, const void* w, int dtype, const int* ids, void* act,
+                    int tokens, int top, int ff, int K, int kind, float limit, float alpha,
+                    float beta, hipStream_t stream);
+int mk_expert_down(const void* act, const void* w, int dtype, const int* ids, const float* weights,
+                   float* y, int tokens, int top, int ff, int N, hipStream_t stream);
+
+// out[t, i] = gate_act(gate_up[t, i], gate_up[t, I + i]) for an activation MK_ACT_*.
+int mk_gate_act(const void* gate_up, void* out, int dtype, int tokens, int inter, int kind,
+                float limit, float alpha, float beta, hipStream_t stream);
+
+// h[i] += mult * (y[i] + sum_k a[k * stride + i] + sum_k b[k * stride + i]) for i < n; y may
+// be null.  mk_fill_zero: p[i] = 0 by a kernel (a captured graph records no memset node).
+int mk_scaled_add(float* h, const float* y, const float* a, int na, const float* b, int nb,
+                  long long stride, float mult, long long n, hipStream_t stream);
+int mk_fill_zero(float* p, long long n, hipStream_t stream);
 
 // @library mfma: bfloat16 kernels on the matrix cores
 

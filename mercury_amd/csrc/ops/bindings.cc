@@ -38,6 +38,16 @@ py::bytes blob(const P& params) {
   return py::bytes(reinterpret_cast<const char*>(&params), sizeof params);
 }
 
+GateAct act_from(int kind, float limit, float alpha, float beta) {
+  if (kind != 0 && kind != 1) throw KernelError("unknown gate activation " + std::to_string(kind));
+  GateAct a;
+  a.kind = kind;
+  a.limit = limit;
+  a.alpha = alpha;
+  a.beta = beta;
+  return a;
+}
+
 py::dict plan_to_py(const AttentionPlan& p) {
   py::dict d;
   d["mfma"] = p.mfma;
@@ -220,13 +230,97 @@ void bind_ops(py::module_& m) {
     p.distance_slopes = ptr_of<const float>(d, "distance_slopes");
     return blob(p);
   });
-  m.def("gated_mlp_params", [](uintptr_t w_gate_up, uintptr_t w_down, int inter) {
+  m.def("gated_mlp_params", [](uintptr_t w_gate_up, uintptr_t w_down, int inter, int act,
+                                float limit, float alpha, float beta) {
     GatedMlpParams p;
     p.w_gate_up = as_ptr<const void>(w_gate_up);
     p.w_down = as_ptr<const void>(w_down);
     p.inter = inter;
+    p.act = act_from(act, limit, alpha, beta);
+    return blob(p);
+  }, py::arg("w_gate_up"), py::arg("w_down"), py::arg("inter"), py::arg("act") = 0,
+     py::arg("limit") = 0.f, py::arg("alpha") = 1.f, py::arg("beta") = 0.f);
+  m.def("latent_attention_params", [](const py::kwargs& kw) {
+    const py::dict d = kw;
+    LatentAttentionParams p;
+    LatentArgs& a = p.latent;
+    a.w_down = ptr_of<const void>(d, "w_down");
+    a.q_norm = ptr_of<const void>(d, "q_norm");
+    a.kv_norm = ptr_of<const void>(d, "kv_norm");
+    a.norm_dtype = get<int>(d, "norm_dtype", kF32);
+    a.eps = get<float>(d, "eps", 0.f);
+    a.w_uq = ptr_of<const void>(d, "w_uq");
+    a.w_uk_t = ptr_of<const void>(d, "w_uk_t");
+    a.w_uv = ptr_of<const void>(d, "w_uv");
+    a.heads = get<int>(d, "heads", 0);
+    a.dim = get<int>(d, "dim", 0);
+    a.rot = get<int>(d, "rot", 0);
+    a.vdim = get<int>(d, "vdim", 0);
+    a.q_rank = get<int>(d, "q_rank", 0);
+    a.kv_rank = get<int>(d, "kv_rank", 0);
+    a.pos.rotary_dim = get<int>(d, "rotary_dim", 0);
+    a.pos.cos = ptr_of<const float>(d, "cos");
+    a.pos.sin = ptr_of<const float>(d, "sin");
+    a.pos.table_positions = get<int>(d, "table_positions", 0);
+    a.pos.interleaved = get<bool>(d, "interleaved", false) ? 1 : 0;
+    a.k_cache = ptr_of<void>(d, "k_cache");
+    a.v_cache = ptr_of<void>(d, "v_cache");
+    a.page_size = get<int>(d, "page_size", 1);
+    a.writes = get<bool>(d, "writes", true);
+    p.w_o = ptr_of<const void>(d, "w_o");
+    p.group = get<int>(d, "group", 0);
+    p.window = get<int>(d, "window", 0);
+    p.scale = get<float>(d, "scale", 0.f);
+    if (a.heads <= 0 || a.dim <= 0 || a.vdim <= 0 || a.q_rank <= 0 || a.kv_rank <= 0 || a.rot < 0 ||
+        a.pos.rotary_dim > a.rot) {
+      throw KernelError("latent attention: bad sizes");
+    }
     return blob(p);
   });
+  m.def("routed_experts_params", [](const py::kwargs& kw) {
+    const py::dict d = kw;
+    RoutedExpertsParams p;
+    ExpertArgs& a = p.experts;
+    a.w_router = ptr_of<const void>(d, "w_router");
+    a.w_gate_up = ptr_of<const void>(d, "w_gate_up");
+    a.w_down = ptr_of<const void>(d, "w_down");
+    a.experts = get<int>(d, "experts", 0);
+    a.top = get<int>(d, "top", 0);
+    a.ff = get<int>(d, "ff", 0);
+    a.scale = get<float>(d, "scale", 1.f);
+    a.renormalize = get<bool>(d, "renormalize", false) ? 1 : 0;
+    a.act = act_from(get<int>(d, "act", 0), get<float>(d, "limit", 0.f), get<float>(d, "alpha", 1.f),
+                     get<float>(d, "beta", 0.f));
+    if (a.experts <= 0 || a.top <= 0 || a.top > a.experts || a.ff <= 0) {
+      throw KernelError("routed experts: bad sizes");
+    }
+    return blob(p);
+  });
+  m.def("parallel_params", [](float mult, const std::vector<std::pair<std::string, py::bytes>>& subs) {
+    if (subs.empty() || (int)subs.size() > kParallelMax) {
+      throw KernelError("a parallel layer holds 1 to " + std::to_string(kParallelMax) + " sublayers");
+    }
+    ParallelParams p;
+    p.mult = mult;
+    p.count = (int)subs.size();
+    std::string out(sizeof p, '\0');
+    for (size_t i = 0; i < subs.size(); ++i) {
+      const OpKind& kind = OpRegistry::instance().get(subs[i].first);
+      if (kind.flags & MK_OP_FOLDS_PENDING) {
+        throw KernelError("a sublayer of a parallel layer cannot be an operation that adds up partial sums");
+      }
+      const std::string bytes = subs[i].second;
+      out.resize((out.size() + 15) / 16 * 16, '\0');
+      p.sub[i].run = kind.run;
+      p.sub[i].tiles = kind.tiles;
+      p.sub[i].flags = kind.flags;
+      p.sub[i].offset = (int)out.size();
+      out += bytes;
+    }
+    std::memcpy(&out[0], &p, sizeof p);
+    return py::bytes(out);
+  }, py::arg("mult"), py::arg("sublayers"),
+     "The parameter block of a 'parallel' operation: sublayers as (kind, parameter bytes).");
   m.def("head_params", [](uintptr_t weight, uintptr_t bias, int bias_dtype, float cap) {
     HeadParams p;
     p.weight = as_ptr<const void>(weight);

@@ -142,7 +142,8 @@ int run_gated_mlp(const void* params, mk_op_context* ctx) {
     if (ctx->x_rows != m) throw KernelError("the gated projection reads an x of every token");
     Launch l(ctx);
     NormFold fold;
-    const void* act = gated(l, ctx->x, m, ctx->hidden, p.w_gate_up, p.inter, -2, fold_of(ctx, fold));
+    const void* act = gated(l, ctx->x, m, ctx->hidden, p.w_gate_up, p.inter, -2, fold_of(ctx, fold),
+                            p.act);
     if (ctx->stream_fixed) {
       project_into_fixed(l, act, m, p.w_down, ctx->hidden, p.inter, nullptr, kF32, ctx->h_fixed);
       return;
@@ -150,6 +151,98 @@ int run_gated_mlp(const void* params, mk_op_context* ctx) {
     project_into_stream(l, act, m, p.w_down, ctx->hidden, p.inter, nullptr, kF32, ctx->h,
                         ctx->out_pending, ctx->out_pending_count);
   });
+}
+
+int run_latent_attention(const void* params, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    const LatentAttentionParams& p = *static_cast<const LatentAttentionParams*>(params);
+    const LatentArgs& a = p.latent;
+    const mk_step_view& s = *ctx->step;
+    if (ctx->x_rows != s.num_tokens) throw KernelError("attention reads an x of every token");
+    Launch l(ctx);
+    const StepArrays arrays = arrays_of(s, p.group);
+    const Queries q = latent_queries(l, ctx->x, s.num_tokens, ctx->hidden, a, arrays);
+    AttendArgs at;
+    at.n_q = a.heads;
+    at.n_kv = 1;
+    at.head_dim = a.key_width();
+    at.value_dim = a.kv_rank;
+    at.page_size = a.page_size;
+    at.window = p.window;
+    at.scale = p.scale;
+    at.k_cache = a.k_cache;
+    at.v_cache = a.v_cache;
+    const void* summed = attend(l, q, at, arrays, s);
+    const void* values = latent_values(l, summed, s.num_tokens, a);
+    project_into_stream(l, values, s.num_tokens, p.w_o, ctx->hidden, a.heads * a.vdim, nullptr, kF32,
+                        ctx->h, ctx->out_pending, ctx->out_pending_count);
+  });
+}
+
+int run_routed_experts(const void* params, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    const RoutedExpertsParams& p = *static_cast<const RoutedExpertsParams*>(params);
+    const int m = ctx->step->num_tokens;
+    if (ctx->x_rows != m) throw KernelError("the experts read an x of every token");
+    Launch l(ctx);
+    routed_experts(l, ctx->x, m, ctx->hidden, p.experts, ctx->h);
+  });
+}
+
+int run_parallel(const void* params, mk_op_context* ctx) {
+  const ParallelParams& p = *static_cast<const ParallelParams*>(params);
+  const long long n = (long long)ctx->step->num_tokens * ctx->hidden;
+  float* const h = ctx->h;
+  float* y = nullptr;
+  int code = guarded(ctx, [&] {
+    Launch l(ctx);
+    y = zeros(l, n);
+  });
+  if (code) return code;
+  const float* parts[kParallelMax] = {nullptr};
+  int counts[kParallelMax] = {0};
+  for (int i = 0; i < p.count; ++i) {
+    ctx->h = y;
+    ctx->out_x = nullptr;
+    ctx->out_x_rows = ctx->out_x_live = 0;
+    ctx->out_pending = nullptr;
+    ctx->out_pending_count = 0;
+    code = p.sub[i].run(static_cast<const char*>(params) + p.sub[i].offset, ctx);
+    ctx->h = h;
+    if (code) return code;
+    parts[i] = ctx->out_pending;
+    counts[i] = ctx->out_pending_count;
+  }
+  ctx->out_x = nullptr;
+  ctx->out_x_rows = ctx->out_x_live = 0;
+  ctx->out_pending = nullptr;
+  ctx->out_pending_count = 0;
+  ctx->out_logits_ready = 0;
+  return guarded(ctx, [&] {
+    Launch l(ctx);
+    // partial sums of at most two sublayers go into the sum directly; any further ones first
+    // into y
+    int first = -1, second = -1;
+    for (int i = 0; i < p.count; ++i) {
+      if (!counts[i]) continue;
+      if (first < 0) first = i;
+      else if (second < 0) second = i;
+      else scaled_add(l, y, nullptr, parts[i], counts[i], nullptr, 0, n, 1.f);
+    }
+    scaled_add(l, h, y, first < 0 ? nullptr : parts[first], first < 0 ? 0 : counts[first],
+               second < 0 ? nullptr : parts[second], second < 0 ? 0 : counts[second], n, p.mult);
+  });
+}
+
+int tiles_parallel(const void* params, const mk_step_shape* shape, mk_tile_need* out) {
+  const ParallelParams& p = *static_cast<const ParallelParams*>(params);
+  for (int i = 0; i < p.count; ++i) {
+    if (p.sub[i].tiles &&
+        p.sub[i].tiles(static_cast<const char*>(params) + p.sub[i].offset, shape, out) > 0) {
+      return 1;
+    }
+  }
+  return 0;
 }
 
 int run_head(const void* params, mk_op_context* ctx) {
@@ -174,6 +267,9 @@ void register_builtin_ops() {
   r.add(OpKind{"norm", &run_norm, nullptr, MK_OP_FOLDS_PENDING | MK_OP_FIXED_STREAM});
   r.add(OpKind{"attention", &run_attention, &tiles_attention, MK_OP_READS_X | MK_OP_FIXED_STREAM});
   r.add(OpKind{"gated_mlp", &run_gated_mlp, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
+  r.add(OpKind{"latent_attention", &run_latent_attention, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"routed_experts", &run_routed_experts, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"parallel", &run_parallel, &tiles_parallel, MK_OP_READS_X});
   r.add(OpKind{"head", &run_head, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
   r.fixed_stream_tokens = &fixed_stream_tokens;
 }

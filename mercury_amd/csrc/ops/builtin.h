@@ -40,6 +40,38 @@ struct AttentionParams {
 struct GatedMlpParams {
   const void *w_gate_up = nullptr, *w_down = nullptr;
   int inter = 0;
+  GateAct act;
+};
+
+// "latent_attention": attention through a low-rank latent shared by the heads (launch.h),
+// its output projection into h (or left as partial sums).
+struct LatentAttentionParams {
+  LatentArgs latent;
+  const void* w_o = nullptr;   // [hidden, heads vdim]
+  int group = 0;               // which of the step's block tables
+  int window = 0;
+  float scale = 0.f;
+};
+
+// "routed_experts": h += sum over a token's chosen experts (launch.h).
+struct RoutedExpertsParams {
+  ExpertArgs experts;
+};
+
+// "parallel": sublayers that read the same x, their outputs summed, scaled and added:
+// h += mult * (f_0(x) + f_1(x) ...).  Each sublayer is an operation of a registered kind that
+// adds its output into h; here it gets a zeroed buffer in h's place.  The block is this header
+// followed by the sublayers' parameter blocks at `offset` bytes from its start.
+constexpr int kParallelMax = 4;
+struct ParallelParams {
+  float mult = 1.f;
+  int count = 0;
+  struct Sub {
+    mk_op_run_fn run = nullptr;
+    mk_op_tiles_fn tiles = nullptr;
+    int flags = 0;
+    int offset = 0;
+  } sub[kParallelMax];
 };
 
 // "head": logits = x W^T (+ bias), optionally capped to cap * tanh(. / cap).

@@ -66,6 +66,28 @@ void* silu_mul(Launch& l, const void* gate_up, int tokens, int inter, void* out)
   return out;
 }
 
+void* gate_activation(Launch& l, const void* gate_up, int tokens, int inter, const GateAct& act,
+                      void* out) {
+  if (!out) out = l.alloc((size_t)tokens * inter * l.elem());
+  if (l.dry() || tokens == 0) return out;
+  check_core(need_core().mk_gate_act(gate_up, out, l.dtype(), tokens, inter, act.kind, act.limit,
+                                     act.alpha, act.beta, l.stream()), "gate_activation");
+  return out;
+}
+
+void scaled_add(Launch& l, float* h, const float* y, const float* a, int na, const float* b, int nb,
+                long long n, float mult) {
+  if (l.dry() || n == 0) return;
+  check_core(need_core().mk_scaled_add(h, y, a, na, b, nb, n, mult, n, l.stream()), "scaled_add");
+}
+
+float* zeros(Launch& l, long long n) {
+  float* p = (float*)l.alloc((size_t)n * 4);
+  if (l.dry() || n == 0) return p;
+  check_core(need_core().mk_fill_zero(p, n, l.stream()), "zeros");
+  return p;
+}
+
 void logit_cap(Launch& l, float* logits, long long count, float cap) {
   if (l.dry() || count == 0) return;
   check_core(need_core().mk_logit_cap(logits, count, cap, l.stream()), "logit_cap");
@@ -223,6 +245,12 @@ AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
     }
     return AttentionPlan();     // the float32-arithmetic kernel
   }
+  if (a.v_dim() != a.head_dim) {
+    if (force.kernel == 2) {
+      throw KernelError("attention: the matrix-core kernels keep values as wide as keys");
+    }
+    return AttentionPlan();
+  }
   const std::vector<int> counts(step.counts, step.counts + step.num_seqs);
   return plan_attention(dtype, a.head_dim, a.page_size, a.n_q, a.n_kv, a.window, counts,
                         step.max_q_len, step.max_kv_len, force.kernel, force.tile_rows, force.staged,
@@ -243,14 +271,15 @@ const mk_tile_list& tiles_for(const mk_step_view& step, int group, int tile_rows
 void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
              const mk_step_view& step, AttendForce force, void* out) {
   const int m = step.num_tokens, d = a.head_dim;
-  if (!out) out = l.alloc((size_t)m * a.n_q * d * l.elem());
+  if (!out) out = l.alloc((size_t)m * a.n_q * a.v_dim() * l.elem());
   const AttentionPlan plan = plan_for(l.dtype(), a, step, force);
   if (!plan.mfma) {
     if (!l.dry() && m > 0) {
-      check_core(need_core().mk_attention_generic(
-                     q.q, q.stride, out, a.n_q * d, a.k_cache, a.v_cache, l.dtype(), s.positions,
-                     s.token_seq, s.table, s.table_stride, a.page_size, a.n_q, a.n_kv, d, a.scale,
-                     a.window, a.score_cap, a.distance_slopes, m, l.stream()), "attention");
+      check_core(need_core().mk_attention_generic_kv(
+                     q.q, q.stride, out, a.n_q * a.v_dim(), a.k_cache, a.v_cache, l.dtype(),
+                     s.positions, s.token_seq, s.table, s.table_stride, a.page_size, a.n_q, a.n_kv,
+                     d, a.v_dim(), a.scale, a.window, a.score_cap, a.distance_slopes, m,
+                     l.stream()), "attention");
     }
     return out;
   }
@@ -342,8 +371,8 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
 }
 
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
-            int tile_config, const NormFold* fold) {
-  const bool fuses = fuses_gating(l.dtype(), l.dtype(), m, k, 2 * inter);
+            int tile_config, const NormFold* fold, const GateAct& act) {
+  const bool fuses = act.silu() && fuses_gating(l.dtype(), l.dtype(), m, k, 2 * inter);
   const bool folded = fold && fuses && tile_config == -2 && m <= 16 && folds_norm(l.dtype(), m, k);
   if (fold && !folded) {
     x = rmsnorm_fixed(l, fold->h64, k, fold->weight, fold->weight_dtype, fold->eps, nullptr, m);
@@ -367,7 +396,73 @@ void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int i
   }
   if (tile_config != -2) throw KernelError("gated_projection: operands not eligible");
   void* gate_up = linear(l, x, m, w_gate_up, 2 * inter, k, nullptr, kF32, nullptr, l.dtype(), false);
-  return silu_mul(l, gate_up, m, inter);
+  return act.silu() ? silu_mul(l, gate_up, m, inter) : gate_activation(l, gate_up, m, inter, act);
+}
+
+void* linear_per_head(Launch& l, const void* x, int m, int heads, int lda, int x_head,
+                      const void* w, int n, int k, void* out, int ldo, int o_head) {
+  if (!out) {
+    out = l.alloc((size_t)m * heads * n * l.elem());
+    ldo = heads * n;
+    o_head = n;
+  }
+  if (l.dry() || m == 0) return out;
+  check_core(need_core().mk_linear_batched_generic(x, w, l.dtype(), out, l.dtype(), m, n, k, lda,
+                                                   ldo, heads, x_head, (long long)n * k, o_head,
+                                                   l.stream()), "linear_per_head");
+  return out;
+}
+
+Queries latent_queries(Launch& l, const void* x, int m, int hidden, const LatentArgs& a,
+                       const StepArrays& s) {
+  const int down_width = a.q_rank + (a.writes ? a.kv_rank + a.rot : 0);
+  const int per_head = a.dim + a.rot, width = a.key_width();
+  // the latents in float32: the norms read them
+  const float* down = (const float*)linear(l, x, m, a.w_down, down_width, hidden, nullptr, kF32,
+                                           nullptr, kF32, false);
+  void* q_latent = l.alloc((size_t)m * a.q_rank * l.elem());
+  if (!l.dry() && m > 0) {
+    check_core(need_core().mk_latent_prepare(
+                   down, down_width, a.q_rank, a.kv_rank, a.rot, a.q_norm, a.kv_norm, a.norm_dtype,
+                   a.eps, a.pos.cos, a.pos.sin, a.pos.table_positions, a.pos.rotary_dim,
+                   a.pos.interleaved, s.positions, s.token_seq, s.table, s.table_stride, q_latent,
+                   a.writes ? a.k_cache : nullptr, a.writes ? a.v_cache : nullptr, l.dtype(),
+                   a.writes ? a.page_size : 1, a.writes ? 1 : 0, m, l.stream()), "latent_prepare");
+  }
+  const void* q = linear(l, q_latent, m, a.w_uq, a.heads * per_head, a.q_rank, nullptr, kF32,
+                         nullptr, l.dtype(), false);
+  void* out = l.alloc((size_t)m * a.heads * width * l.elem());
+  linear_per_head(l, q, m, a.heads, a.heads * per_head, per_head, a.w_uk_t, a.kv_rank, a.dim, out,
+                  a.heads * width, width);
+  if (!l.dry() && m > 0) {
+    check_core(need_core().mk_latent_query_tail(
+                   q, l.dtype(), a.heads, a.dim, a.rot, a.pos.cos, a.pos.sin, a.pos.table_positions,
+                   a.pos.rotary_dim, a.pos.interleaved, s.positions, out, width, a.kv_rank, m,
+                   l.stream()), "latent_query_tail");
+  }
+  return {out, a.heads * width};
+}
+
+void* latent_values(Launch& l, const void* summed, int m, const LatentArgs& a) {
+  return linear_per_head(l, summed, m, a.heads, a.heads * a.kv_rank, a.kv_rank, a.w_uv, a.vdim,
+                         a.kv_rank, nullptr, 0, 0);
+}
+
+void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y) {
+  const float* logits = (const float*)linear(l, x, m, a.w_router, a.experts, hidden, nullptr, kF32,
+                                             nullptr, kF32, false);
+  int* ids = (int*)l.alloc((size_t)m * a.top * 4);
+  float* weights = (float*)l.alloc((size_t)m * a.top * 4);
+  void* act = l.alloc((size_t)m * a.top * a.ff * l.elem());
+  if (l.dry() || m == 0) return;
+  const KernelTable& t = need_core();
+  check_core(t.mk_route_topk(logits, a.experts, a.top, a.scale, a.renormalize, ids, weights, m,
+                             l.stream()), "route");
+  check_core(t.mk_expert_gated(x, a.w_gate_up, l.dtype(), ids, act, m, a.top, a.ff, hidden,
+                               a.act.kind, a.act.limit, a.act.alpha, a.act.beta, l.stream()),
+             "expert_gated");
+  check_core(t.mk_expert_down(act, a.w_down, l.dtype(), ids, weights, y, m, a.top, a.ff, hidden,
+                              l.stream()), "expert_down");
 }
 
 }  // namespace mercury

@@ -52,6 +52,22 @@ void project_into_fixed(Launch& l, const void* x, int m, const void* w, int n, i
 
 void* silu_mul(Launch& l, const void* gate_up, int tokens, int inter, void* out = nullptr);
 
+// The activation of a gated feed-forward with its constants (MK_ACT_* of mercury_kernels.h):
+// silu(g) * u, or g' * sigmoid(alpha g') * (u' + beta) on g' = min(g, limit) and
+// u' = clamp(u, -limit, limit).
+struct GateAct {
+  int kind = 0;
+  float limit = 0.f, alpha = 1.f, beta = 0.f;
+  bool silu() const { return kind == 0; }
+};
+void* gate_activation(Launch& l, const void* gate_up, int tokens, int inter, const GateAct& act,
+                      void* out = nullptr);
+
+// h += mult * (y + the partial sums a [na, n] and b [nb, n]); y may be null.
+void scaled_add(Launch& l, float* h, const float* y, const float* a, int na, const float* b, int nb,
+                long long n, float mult);
+float* zeros(Launch& l, long long n);
+
 // logits <- cap * tanh(logits / cap), in place.
 void logit_cap(Launch& l, float* logits, long long count, float cap);
 
@@ -133,6 +149,8 @@ void* qkv_finish(Launch& l, const float* parts, int slices, int m, const QkvArgs
 
 struct AttendArgs {
   int n_q = 0, n_kv = 0, head_dim = 0, page_size = 0, window = 0;
+  int value_dim = 0;     // 0: values as wide as keys
+  int v_dim() const { return value_dim > 0 ? value_dim : head_dim; }
   float scale = 0.f;
   const void *k_cache = nullptr, *v_cache = nullptr;
   // What only the float32-arithmetic kernel computes: a bound cap * tanh(score / cap) on the
@@ -171,6 +189,51 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
 // sizes, else the tiled kernel with that configuration (-1: its own choice).
 // `fold` as for qkv_project.
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
-            int tile_config = -2, const NormFold* fold = nullptr);
+            int tile_config = -2, const NormFold* fold = nullptr, const GateAct& act = {});
+
+// y[t, head, :] = W[head] x[t, head, :] for every head: x rows `lda` apart with head `head`
+// at x + head * x_head, W [heads, n, k], y rows `ldo` apart with the head at out + head * o_head
+// (elements).  `out` is allocated as [m, heads * n] when null (then ldo = heads * n, o_head = n).
+void* linear_per_head(Launch& l, const void* x, int m, int heads, int lda, int x_head,
+                      const void* w, int n, int k, void* out, int ldo, int o_head);
+
+// Attention through a low-rank latent shared by the heads.  Per token the cache holds one key
+// row [c | r] (c the normed latent of kv_rank, r the rotated key part of `rot`) and c once
+// more as the value; a query head h scores (W_uk[h]^T q_h) . c + rot(q_rot_h) . r, and its
+// output is W_uv[h] applied to the attention's weighted sum of latents.
+struct LatentArgs {
+  const void* w_down = nullptr;    // [q_rank + kv_rank + rot, hidden]: query latent, c, r
+  const void *q_norm = nullptr, *kv_norm = nullptr;
+  int norm_dtype = 0;
+  float eps = 0.f;
+  const void* w_uq = nullptr;      // [heads (dim + rot), q_rank]
+  const void* w_uk_t = nullptr;    // [heads, kv_rank, dim]: W_uk per head, transposed
+  const void* w_uv = nullptr;      // [heads, vdim, kv_rank]
+  int heads = 0, dim = 0, rot = 0, vdim = 0, q_rank = 0, kv_rank = 0;
+  PositionDesc pos;                // over the first pos.rotary_dim dims of the rotated parts
+  void *k_cache = nullptr, *v_cache = nullptr;
+  int page_size = 1;
+  bool writes = true;
+  int key_width() const { return kv_rank + rot; }
+};
+// Down-projection, norms, rotation and cache write, query up-projection; the queries come back
+// as rows [heads, kv_rank + rot] = [absorbed | rotated].
+Queries latent_queries(Launch& l, const void* x, int m, int hidden, const LatentArgs& a,
+                       const StepArrays& s);
+// [m, heads, kv_rank] weighted sums of latents -> [m, heads vdim] values.
+void* latent_values(Launch& l, const void* summed, int m, const LatentArgs& a);
+
+// Routed experts: router logits in float32, the `top` of softmax, and
+// y += sum_j weight_j * down_ej(act(gate_ej x, up_ej x)); y float32 [m, hidden].
+struct ExpertArgs {
+  const void* w_router = nullptr;    // [experts, hidden]
+  const void* w_gate_up = nullptr;   // [experts, 2 ff, hidden]
+  const void* w_down = nullptr;      // [experts, hidden, ff]
+  int experts = 0, top = 0, ff = 0;
+  float scale = 1.f;
+  int renormalize = 0;
+  GateAct act;
+};
+void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y);
 
 }  // namespace mercury

@@ -31,6 +31,8 @@ LIBRARIES = {
         "elementwise.hip",
         "gemm_generic.hip",
         "attention_generic.hip",
+        "latent.hip",
+        "experts.hip",
         "sampling.hip",
         "random_fill.hip",
     ],

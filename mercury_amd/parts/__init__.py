@@ -3,9 +3,11 @@
 from .attention import Attention
 from .base import (CacheSpec, FeedForward, LayerCache, Mixer, Norm, Part, PositionDescriptor,
                    PositionEncoding, StateSpec, TensorSpec)
-from .block import PreNormBlock
+from .block import ParallelBlock, PreNormBlock
 from .embedding import OutputHead, TokenEmbedding
+from .experts import RoutedExperts
 from .feedforward import GatedMLP
+from .latent_attention import LatentAttention
 from .lowering import OneOp
 from .model import CallerStep, DecoderModel, LayerCall, Registers
 from .norm import RMSNorm
@@ -14,16 +16,20 @@ from .registry import (build_part, known, register_block, register_ffn, register
                        register_norm, register_position)
 
 register_mixer("attention")(Attention)
+register_mixer("latent_attention")(LatentAttention)
 register_ffn("gated_mlp")(GatedMLP)
+register_ffn("routed_experts")(RoutedExperts)
 register_norm("rmsnorm")(RMSNorm)
 register_position("rotary")(RotaryPosition)
 register_position("none")(NoPosition)
 register_block("pre_norm")(PreNormBlock)
+register_block("parallel")(ParallelBlock)
 
 __all__ = [
     "Attention", "CacheSpec", "CallerStep", "DecoderModel", "FeedForward", "GatedMLP",
-    "LayerCache", "LayerCall", "Mixer", "NoPosition", "Norm", "OneOp", "OutputHead", "Part",
-    "PositionDescriptor", "PositionEncoding", "PreNormBlock", "Registers",
+    "LatentAttention", "LayerCache", "LayerCall", "Mixer", "NoPosition", "Norm", "OneOp", "OutputHead", "Part",
+    "ParallelBlock", "PositionDescriptor", "PositionEncoding", "PreNormBlock", "Registers",
+    "RoutedExperts",
     "RMSNorm", "RotaryPosition", "StateSpec", "TensorSpec", "TokenEmbedding", "build_part", "known",
     "register_block", "register_ffn", "register_mixer", "register_norm", "register_position",
 ]

@@ -2,7 +2,11 @@
 
 from __future__ import annotations
 
+import torch
+
+from ..hostcore import core
 from .base import FeedForward, Mixer, Norm, Part
+from .lowering import OneOp
 
 
 class PreNormBlock(Part):
@@ -78,3 +82,100 @@ class PreNormBlock(Part):
             x = self.norm_ffn.forward(h, dtype, partials=pending)
             pending = self.ffn.forward(x, step, h)
         return pending
+
+
+class _Recorder:
+    """Stands in for a program while a sublayer lowers itself: keeps what it appends."""
+
+    def __init__(self):
+        self.ops: list = []
+
+    def append(self, kind: str, params: bytes) -> None:
+        self.ops.append((kind, params))
+
+
+class ParallelBlock(Part):
+    """h += mult * (mixer(x) + ffn(x)) with x = norm(h): one norm, both sublayers read its
+    output, and their sum enters the float32 residual stream scaled by `mult`.  `ffn` may be
+    None.
+
+    Lowered, the layer is the norm and one ``parallel`` operation that holds the sublayers'
+    own operations (each must lower itself to exactly one) and runs them on the same x, their
+    outputs going into a buffer in the stream's place.  `names` gives the checkpoint
+    sub-prefix of each part: ``{"mixer": ..., "ffn": ..., "norm": ...}``.
+    """
+
+    def __init__(self, mixer: Mixer, ffn: FeedForward | None, norm: Norm, names: dict,
+                 residual_mult: float = 1.0):
+        self.mixer, self.ffn, self.norm = mixer, ffn, norm
+        self.residual_mult = float(residual_mult)
+        self.names = dict(names)
+        self._alone: dict = {}
+
+    def _children(self):
+        out = [("mixer", self.mixer), ("norm", self.norm)]
+        if self.ffn is not None:
+            out.append(("ffn", self.ffn))
+        return out
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for _, part in self._children())
+
+    def lowerable_with(self, state) -> bool:
+        if state is not None and not getattr(self.mixer, "lowers_state", False):
+            return False
+        return all(part.can_lower() for _, part in self._children())
+
+    def lower(self, program, cache, state=None) -> None:
+        self.norm.lower(program)
+        sub = _Recorder()
+        if state is None:
+            self.mixer.lower(sub, cache)
+        else:
+            self.mixer.lower(sub, cache, state)
+        if self.ffn is not None:
+            self.ffn.lower(sub)
+        if len(sub.ops) != (1 if self.ffn is None else 2):
+            raise ValueError("a sublayer of a parallel block lowers itself to one operation")
+        program.append("parallel", core.parallel_params(self.residual_mult, sub.ops))
+
+    def param_specs(self) -> dict:
+        specs = {}
+        for key, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[self.names[key] + name] = spec
+        return specs
+
+    def bind(self, params, dtype, device) -> None:
+        for key, part in self._children():
+            prefix = self.names[key]
+            part.bind({n[len(prefix):]: t for n, t in params.items() if n.startswith(prefix)},
+                      dtype, device)
+        self._alone.clear()
+
+    def prepare(self, max_positions: int, device) -> None:
+        self.mixer.prepare(max_positions, device)
+
+    def weight_bytes(self) -> int:
+        return sum(part.weight_bytes() for _, part in self._children())
+
+    def forward(self, h, step, cache, state, dtype, pending=None):
+        if self.lowerable_with(state):
+            # the operations `lower` appends, as a program of their own
+            key = (None if cache is None else cache.k.data_ptr(), None if state is None else state.data_ptr())
+            alone = self._alone.get(key)
+            if alone is None:
+                alone = self._alone[key] = OneOp(dtype, h.shape[1], 0,
+                                                 lambda program: self.lower(program, cache, state))
+            _logits, _x, left = alone.run(step, h, pending=pending)
+            return left
+        # a sublayer that stays with Python: the same sum, put together here
+        x = self.norm.forward(h, dtype, partials=pending)
+        y = torch.zeros_like(h)
+        for left in (self.mixer.forward(x, step, cache, state, y),
+                     None if self.ffn is None else self.ffn.forward(x, step, y)):
+            if left is not None:
+                y += left.sum(dim=0)
+        h.add_(y, alpha=self.residual_mult)
+        return None

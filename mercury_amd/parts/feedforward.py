@@ -8,24 +8,35 @@ from ..hostcore import core
 from .base import FeedForward, TensorSpec
 from .lowering import OneOp
 
-ACTIVATIONS = ("silu",)
+ACTIVATIONS = ("silu", "swish_clamp")
+# the kernels' codes of the activations
+ACTIVATION_CODES = {"silu": 0, "swish_clamp": 1}
 DEFAULT_NAMES = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
 
 
 class GatedMLP(FeedForward):
-    """down(act(gate(x)) * up(x)) without biases, act = SiLU
-    (reference: mercury/model/qwen2.py:34-42).  `names` maps gate, up, down to the stored
-    tensors' leaf names (default ``gate_proj``, ``up_proj``, ``down_proj``)."""
+    """down(act(gate(x), up(x))) without biases.  `activation`:
+
+    ``"silu"``: silu(g) * u (reference: mercury/model/qwen2.py:34-42).
+    ``"swish_clamp"``: g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit) and
+    u' = clamp(u, -limit, limit).
+
+    `names` maps gate, up, down to the stored tensors' leaf names (default ``gate_proj``,
+    ``up_proj``, ``down_proj``)."""
 
     graph_safe = True
     lowerable = True
 
     def __init__(self, hidden: int, intermediate: int, activation: str = "silu",
-                 names: dict | None = None):
+                 names: dict | None = None, limit: float = 0.0, alpha: float = 1.0,
+                 beta: float = 0.0):
         if activation not in ACTIVATIONS:
             raise ValueError(f"activation {activation!r} is not implemented; known: {ACTIVATIONS}")
         self.hidden, self.intermediate = int(hidden), int(intermediate)
         self.activation = activation
+        self.limit, self.alpha, self.beta = float(limit), float(alpha), float(beta)
+        if activation == "swish_clamp" and not self.limit > 0:
+            raise ValueError("swish_clamp needs a positive limit")
         self.names = {**DEFAULT_NAMES, **(names or {})}
         self.w_gate_up = self.w_down = None
         self._alone = None
@@ -51,10 +62,10 @@ class GatedMLP(FeedForward):
         return sum(t.numel() * t.element_size() for t in (self.w_gate_up, self.w_down))
 
     def lower(self, program) -> None:
-        if self.activation != "silu":
-            raise ValueError(f"the gated projection's kernels compute silu, not {self.activation}")
         program.append("gated_mlp", core.gated_mlp_params(
-            self.w_gate_up.data_ptr(), self.w_down.data_ptr(), self.intermediate))
+            self.w_gate_up.data_ptr(), self.w_down.data_ptr(), self.intermediate,
+            act=ACTIVATION_CODES[self.activation], limit=self.limit, alpha=self.alpha,
+            beta=self.beta))
 
     def forward(self, x, step, accum):
         # the operations `lower` appends, as a program of their own

@@ -67,9 +67,18 @@ class DecoderModel(Part):
                  embed_name: str = "model.embed_tokens.weight",
                  norm_prefix: str = "model.norm.", head_name: str = "lm_head.weight",
                  max_positions: int = 0, eos_token_ids: tuple = (), config=None,
-                 embedding: Part | None = None, head: Part | None = None):
+                 embedding: Part | None = None, head: Part | None = None,
+                 layer_ids: list | None = None, stored_name=None):
+        """`layer_ids`: the index each layer's tensors are stored under (default: its place in
+        `layers`), for a model some of whose executed layers own no tensors.  `stored_name`:
+        a function from a tensor's name as the parts compose it (prefixes + the part's leaf,
+        e.g. ``...norm.weight``) to the name the checkpoint stores it under."""
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.layers = list(layers)
+        self.layer_ids = list(layer_ids) if layer_ids is not None else list(range(len(self.layers)))
+        if len(self.layer_ids) != len(self.layers):
+            raise ValueError("one stored index per layer")
+        self.stored_name = stored_name
         self.final_norm = final_norm
         self.tied_head = bool(tied_head)
         self.calls = list(calls) if calls is not None else [
@@ -120,9 +129,18 @@ class DecoderModel(Part):
         return {self.head_name} if self.tied_head else set()
 
     def param_specs(self) -> dict:
+        specs = self._composed_specs()
+        if self.stored_name is None:
+            return specs
+        stored = {self.stored_name(name): spec for name, spec in specs.items()}
+        if len(stored) != len(specs):
+            raise ValueError("two tensors of the model are stored under one name")
+        return stored
+
+    def _composed_specs(self) -> dict:
         specs = {self.embed_prefix + name: spec
                  for name, spec in self.embedding_part.param_specs().items()}
-        for i, layer in enumerate(self.layers):
+        for i, layer in zip(self.layer_ids, self.layers):
             prefix = self.layer_prefix.format(i)
             for name, spec in layer.param_specs().items():
                 specs[prefix + name] = spec
@@ -134,6 +152,9 @@ class DecoderModel(Part):
 
     def bind(self, params, dtype, device) -> None:
         self.dtype = dtype
+        if self.stored_name is not None:
+            composed = {self.stored_name(name): name for name in self._composed_specs()}
+            params = {composed[stored]: t for stored, t in params.items()}
         under = lambda prefix: {n[len(prefix):]: t for n, t in params.items() if n.startswith(prefix)}
         self.embedding_part.bind(under(self.embed_prefix), dtype, device)
         self.embedding = params[self.embed_name]
@@ -142,7 +163,7 @@ class DecoderModel(Part):
             head_params["weight"] = self.embedding
         self.head_part.bind(head_params, dtype, device)
         self.head = head_params["weight"]
-        for i, layer in enumerate(self.layers):
+        for i, layer in zip(self.layer_ids, self.layers):
             layer.bind(under(self.layer_prefix.format(i)), dtype, device)
         self.final_norm.bind(under(self.norm_prefix), dtype, device)
 
