@@ -1,0 +1,291 @@
+// Causal attention of many query heads over ONE shared key/value head whose keys are wider
+// than its values, on the matrix cores (bfloat16 in, float32 accumulate): the attention of a
+// mixer that caches a low-rank latent per token.  A cached token is a key row [c | r] of DK
+// dims and the value c of DV dims, stored once more transposed within the page
+// ([page, DV, slot]) because the value-side product wants the keys as its fast index.
+//
+// Work is cut into tiles of 16 rows, a row being a (token, head) pair of one sequence: row f
+// stands for token f / H and head f % H, so a decoded token's heads share every load of the
+// cache, and a prompt portion of n tokens is ceil(n H / 16) tiles.  A wavefront owns one
+// (tile, part of the keys) and needs no shared memory:
+//
+//   S^T[key, row]  = K[key, :] . Q[row, :]        v_mfma_f32_16x16x32_bf16, A = K, B = Q^T
+//   online softmax over keys in float32, base 2 (a lane holds 8 keys of one row)
+//   O^T[dim, row] += V^T[dim, key] P^T[key, row]  A = V^T, B = P^T
+//
+// The first product leaves a lane with the probabilities the second wants from it as B.
+// Widths are multiples of 32 (keys) and 16 (values): the cache rows and the queries are
+// padded with zeros by whoever writes them.  The counts of 32-wide key chunks and 16-wide
+// value tiles are run-time numbers below a compile-time bound (MAXC, MAXT), which sizes the
+// register arrays; four bounds are compiled.  With the keys split into parts, every part
+// leaves an unnormalised result with its running maximum and sum, and a second kernel merges
+// the parts in order.
+#include "common.h"
+#include "mercury_kernels.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+union LFrag {
+  bf16x8 v;
+  uint4 u;
+  uint2 u2[2];
+};
+
+struct LatentAttnParams {
+  const bf16_t* q;       // [T, heads, dkc * 32]
+  bf16_t* out;           // [T, heads * dv]
+  float* part_o;         // [tile, part, dvt * 16, 16]
+  float* part_ml;        // [tile, part, 2, 16]
+  const bf16_t* k_cache; // [pages, page, dkc * 32]
+  const bf16_t* v_cache; // [pages, dvt * 16, page]
+  const int* tile_seq;
+  const int* tile_row0;
+  const int* cu_q;
+  const int* kv_len;
+  const int* block_table;
+  int table_stride;
+  int page_shift;
+  int heads;
+  int dkc, dvt, dv;
+  float scale_log2;      // scale * log2(e)
+  int num_tiles;
+  int num_parts;
+};
+
+#define LAT_WAVES 4
+
+template <int MAXC, int MAXT>
+__global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnParams p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = blockIdx.x * LAT_WAVES + wave;
+  if (unit >= p.num_tiles * p.num_parts) return;   // a whole wavefront; nothing is shared
+  // Tiles from the last: under a causal mask the later tiles of a prompt read the most keys.
+  const int tile = p.num_tiles - 1 - unit / p.num_parts;
+  const int part = unit % p.num_parts;
+  const int r = lane & 15, g4 = lane >> 4;
+  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
+  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  const int kv_len = p.kv_len[seq];
+  const int rows = q_len * p.heads;
+  const int f = min(row0 + r, rows - 1);            // a row past the end repeats the last one
+  const bool row_ok = row0 + r < rows;
+  const int token = q0 + f / p.heads, head = f % p.heads;
+  const int pos = kv_len - q_len + f / p.heads;
+  const int last_row = min(row0 + 15, rows - 1);
+  const int kmax = kv_len - q_len + last_row / p.heads;       // the tile's last visible key
+  const int all_see = kv_len - q_len + row0 / p.heads;         // keys every row of it sees
+  const int blocks = (kmax >> 5) + 1;
+  const int per = (blocks + p.num_parts - 1) / p.num_parts;
+  const int b_begin = part * per, b_end = min(blocks, b_begin + per);
+  const int ps = 1 << p.page_shift;
+  const int dkp = p.dkc * 32, dvp = p.dvt * 16;
+  const int* table = p.block_table + (size_t)seq * p.table_stride;
+
+  LFrag qf[MAXC];
+  {
+    const bf16_t* qrow = p.q + ((size_t)token * p.heads + head) * dkp + g4 * 8;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c)
+      if (c < p.dkc) qf[c].u = *(const uint4*)(qrow + c * 32);
+  }
+  f32x4 acc[MAXT];
+#pragma unroll
+  for (int t = 0; t < MAXT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+  const float c2 = p.scale_log2;
+
+  for (int b = b_begin; b < b_end; ++b) {
+    const int key0 = b << 5;
+    const bf16_t* kbase[2];
+    const bf16_t* vbase[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int kh = key0 + h * 16;
+      const int index = kh >> p.page_shift;
+      // a half past the sequence's pages reads page 0, which exists; its keys are masked
+      const int page = index < p.table_stride ? max(table[index], 0) : 0;
+      const int off = kh & (ps - 1);
+      kbase[h] = p.k_cache + ((size_t)page * ps + off + r) * dkp + g4 * 8;
+      vbase[h] = p.v_cache + ((size_t)page * dvp + r) * ps + off + g4 * 4;
+    }
+    float s[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < MAXC; ++c) {
+        if (c < p.dkc) {
+          LFrag kf;
+          kf.u = *(const uint4*)(kbase[h] + c * 32);
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sc, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[h * 4 + i] = sc[i];
+    }
+    if (key0 + 31 > all_see) {   // the block holds keys some row does not see
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (key0 + h * 16 + g4 * 4 + i > pos) s[h * 4 + i] = -INFINITY;
+    }
+    float bm = c2 * fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                          fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+      bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+      const float m_new = fmaxf(m, bm);
+      const float corr = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
+      lsum *= corr;
+#pragma unroll
+      for (int t = 0; t < MAXT; ++t) acc[t] *= corr;
+      m = m_new;
+    }
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], c2, -m_use));
+    lsum += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+    LFrag pf;
+    pf.u = make_uint4(pack_bf16x2(e[0], e[1]), pack_bf16x2(e[2], e[3]), pack_bf16x2(e[4], e[5]),
+                      pack_bf16x2(e[6], e[7]));
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) {
+      if (t < p.dvt) {
+        LFrag vf;
+        vf.u2[0] = *(const uint2*)(vbase[0] + (size_t)t * 16 * ps);
+        vf.u2[1] = *(const uint2*)(vbase[1] + (size_t)t * 16 * ps);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  // a row's sum lies in its four lanes
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+
+  if (p.num_parts == 1) {
+    if (!row_ok) return;
+    const float inv = 1.f / lsum;
+    bf16_t* dst = p.out + ((size_t)token * p.heads + head) * p.dv;
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) {
+      if (t < p.dvt) {
+        const int d = t * 16 + g4 * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (d + i < p.dv) dst[d + i] = f32_to_bf16(acc[t][i] * inv);
+      }
+    }
+    return;
+  }
+  // [tile, part, dim, row]: a lane's four dims of its row
+  float* po = p.part_o + ((size_t)tile * p.num_parts + part) * dvp * 16;
+#pragma unroll
+  for (int t = 0; t < MAXT; ++t) {
+    if (t < p.dvt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) po[(size_t)(t * 16 + g4 * 4 + i) * 16 + r] = acc[t][i];
+    }
+  }
+  if (g4 == 0) {
+    float* ml = p.part_ml + ((size_t)tile * p.num_parts + part) * 32;
+    ml[r] = m;
+    ml[16 + r] = lsum;
+  }
+}
+
+// One workgroup per tile: the parts' results added up in part order.
+__global__ __launch_bounds__(256) void attn_latent_merge_kernel(LatentAttnParams p) {
+  __shared__ float weight[64][16];   // at most 64 parts
+  __shared__ float inv[16];
+  const int tile = blockIdx.x;
+  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
+  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  const int rows = q_len * p.heads;
+  const int dvp = p.dvt * 16;
+  const float* ml = p.part_ml + (size_t)tile * p.num_parts * 32;
+  if (threadIdx.x < 16) {
+    const int r = threadIdx.x;
+    float m = -INFINITY;
+    for (int s = 0; s < p.num_parts; ++s) m = fmaxf(m, ml[s * 32 + r]);
+    float total = 0.f;
+    for (int s = 0; s < p.num_parts; ++s) {
+      const float ms = ml[s * 32 + r];
+      const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m);
+      weight[s][r] = w;
+      total += w * ml[s * 32 + 16 + r];
+    }
+    inv[r] = 1.f / total;
+  }
+  __syncthreads();
+  const float* po = p.part_o + (size_t)tile * p.num_parts * dvp * 16;
+  for (int idx = threadIdx.x; idx < dvp * 16; idx += blockDim.x) {
+    const int d = idx >> 4, r = idx & 15;
+    if (row0 + r >= rows || d >= p.dv) continue;
+    float total = 0.f;
+    for (int s = 0; s < p.num_parts; ++s) total += weight[s][r] * po[(size_t)s * dvp * 16 + idx];
+    const int f = row0 + r;
+    p.out[((size_t)(q0 + f / p.heads) * p.heads + f % p.heads) * p.dv + d] =
+        f32_to_bf16(total * inv[r]);
+  }
+}
+
+extern "C" int mk_attention_latent_supported(int dk, int dv, int page_size) {
+  return dk > 0 && dv > 0 && dk % 32 == 0 && dv <= dk && (dv + 15) / 16 <= 32 && dk / 32 <= 18 &&
+         page_size >= 16 && mk_is_pow2(page_size);
+}
+
+extern "C" int mk_attention_latent_max_parts(void) { return 64; }
+
+extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache,
+                                   const void* v_cache, const int* tile_seq, const int* tile_row0,
+                                   int num_tiles, const int* cu_q, const int* kv_len,
+                                   const int* block_table, int table_stride, int page_size,
+                                   int heads, int dk, int dv, float scale, int num_parts,
+                                   float* part_o, float* part_ml, hipStream_t stream) {
+  MK_REQUIRE(mk_attention_latent_supported(dk, dv, page_size),
+             "latent attention: keys of %d, values of %d, pages of %d are not taken", dk, dv,
+             page_size);
+  MK_REQUIRE(heads > 0 && num_tiles >= 0 && table_stride > 0, "latent attention: bad sizes");
+  MK_REQUIRE(num_parts >= 1 && num_parts <= 64, "latent attention: %d parts", num_parts);
+  MK_REQUIRE(num_parts == 1 || (part_o && part_ml), "latent attention: parts without a workspace");
+  MK_REQUIRE(q && out && k_cache && v_cache && tile_seq && tile_row0 && cu_q && kv_len && block_table,
+             "latent attention: null argument");
+  if (num_tiles == 0) return 0;
+  LatentAttnParams p;
+  p.q = (const bf16_t*)q;
+  p.out = (bf16_t*)out;
+  p.part_o = part_o;
+  p.part_ml = part_ml;
+  p.k_cache = (const bf16_t*)k_cache;
+  p.v_cache = (const bf16_t*)v_cache;
+  p.tile_seq = tile_seq;
+  p.tile_row0 = tile_row0;
+  p.cu_q = cu_q;
+  p.kv_len = kv_len;
+  p.block_table = block_table;
+  p.table_stride = table_stride;
+  p.page_shift = mk_log2(page_size);
+  p.heads = heads;
+  p.dkc = dk / 32;
+  p.dvt = (dv + 15) / 16;
+  p.dv = dv;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  p.num_tiles = num_tiles;
+  p.num_parts = num_parts;
+  const long long units = (long long)num_tiles * num_parts;
+  MK_REQUIRE((units + LAT_WAVES - 1) / LAT_WAVES < (1ll << 31), "latent attention: too many tiles");
+  const dim3 grid((unsigned)((units + LAT_WAVES - 1) / LAT_WAVES));
+  if (p.dkc <= 3 && p.dvt <= 4) attn_latent_kernel<3, 4><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
+  else if (p.dkc <= 6 && p.dvt <= 8) attn_latent_kernel<6, 8><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
+  else if (p.dkc <= 10 && p.dvt <= 16) attn_latent_kernel<10, 16><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
+  else attn_latent_kernel<18, 32><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
+  MK_LAUNCH_CHECK("attention_latent");
+  if (num_parts > 1) {
+    attn_latent_merge_kernel<<<num_tiles, 256, 0, stream>>>(p);
+    MK_LAUNCH_CHECK("attention_latent_merge");
+  }
+  return 0;
+}

@@ -108,6 +108,65 @@ extern "C" int mk_route_topk(const float* logits, int experts, int top, float sc
   return 0;
 }
 
+// Pairs grouped by expert, by one workgroup: a histogram in LDS, its prefix sums, and every
+// pair placed at its expert's cursor.  The order within an expert is whatever the atomics
+// give; nothing downstream depends on it (each pair's result goes to the pair's own row).
+#define GROUP_MAX_EXPERTS 1024
+
+__global__ __launch_bounds__(1024) void route_group_kernel(const int* __restrict__ ids, int pairs,
+                                                           int experts, int* __restrict__ rows,
+                                                           int* __restrict__ offsets) {
+  __shared__ int counts[GROUP_MAX_EXPERTS];
+  __shared__ int cursor[GROUP_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) atomicAdd(&counts[ids[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      offsets[e] = at;
+      cursor[e] = at;
+      at += counts[e];
+    }
+    offsets[experts] = at;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) rows[atomicAdd(&cursor[ids[i]], 1)] = i;
+}
+
+extern "C" int mk_route_group(const int* ids, int pairs, int experts, int* rows, int* offsets,
+                              hipStream_t stream) {
+  MK_REQUIRE(pairs >= 0 && experts > 0 && experts <= GROUP_MAX_EXPERTS, "route_group: bad sizes");
+  route_group_kernel<<<1, 1024, 0, stream>>>(ids, pairs, experts, rows, offsets);
+  MK_LAUNCH_CHECK("route_group");
+  return 0;
+}
+
+__global__ void expert_combine_kernel(const float* __restrict__ pairs_out, float* __restrict__ y,
+                                      int top, int N, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / N;
+    const int n = (int)(idx - t * N);
+    float v = 0.f;
+    for (int j = 0; j < top; ++j) v += pairs_out[(t * top + j) * N + n];
+    y[idx] += v;
+  }
+}
+
+extern "C" int mk_expert_combine(const float* pairs_out, float* y, int tokens, int top, int N,
+                                 hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && top > 0 && N > 0, "expert_combine: bad sizes");
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * N;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  expert_combine_kernel<<<(int)blocks, 256, 0, stream>>>(pairs_out, y, top, N, total);
+  MK_LAUNCH_CHECK("expert_combine");
+  return 0;
+}
+
 // ------------------------------------------------------------------- experts, token by token
 
 #define EXPERT_ROWS_PER_WAVE 4
@@ -147,24 +206,33 @@ template <typename T>
 __global__ __launch_bounds__(256) void expert_down_kernel(
     const T* __restrict__ act, const T* __restrict__ w, const int* __restrict__ ids,
     const float* __restrict__ weights, float* __restrict__ y, int top, int ff, int N) {
-  extern __shared__ float as[];   // the token's `top` rows of activations
+  extern __shared__ float as[];   // one row of the token's activations at a time
   const int t = blockIdx.x;
-  const T* ar = act + (size_t)t * top * ff;
-  for (int i = threadIdx.x; i < top * ff; i += blockDim.x) as[i] = Elem<T>::load(ar + i);
-  __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float total[EXPERT_ROWS_PER_WAVE];
+#pragma unroll
+  for (int r = 0; r < EXPERT_ROWS_PER_WAVE; ++r) total[r] = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const T* ar = act + ((size_t)t * top + j) * ff;
+    __syncthreads();
+    for (int i = threadIdx.x; i < ff; i += blockDim.x) as[i] = Elem<T>::load(ar + i);
+    __syncthreads();
+    const float weight = weights[(size_t)t * top + j];
+    const T* we = w + (size_t)ids[(size_t)t * top + j] * N * ff;
+#pragma unroll
+    for (int r = 0; r < EXPERT_ROWS_PER_WAVE; ++r) {
+      const int n = (blockIdx.y * 4 + wave) * EXPERT_ROWS_PER_WAVE + r;
+      if (n >= N) break;
+      const T* wr = we + (size_t)n * ff;
+      float dot = 0.f;
+      for (int i = lane; i < ff; i += MK_WAVE) dot = fmaf(as[i], Elem<T>::load(wr + i), dot);
+      total[r] = fmaf(weight, wave_sum(dot), total[r]);
+    }
+  }
 #pragma unroll
   for (int r = 0; r < EXPERT_ROWS_PER_WAVE; ++r) {
     const int n = (blockIdx.y * 4 + wave) * EXPERT_ROWS_PER_WAVE + r;
-    if (n >= N) break;
-    float total = 0.f;
-    for (int j = 0; j < top; ++j) {
-      const T* wr = w + ((size_t)ids[(size_t)t * top + j] * N + n) * ff;
-      float dot = 0.f;
-      for (int i = lane; i < ff; i += MK_WAVE) dot = fmaf(as[j * ff + i], Elem<T>::load(wr + i), dot);
-      total = fmaf(weights[(size_t)t * top + j], wave_sum(dot), total);
-    }
-    if (lane == 0) y[(size_t)t * N + n] += total;
+    if (n < N && lane == 0) y[(size_t)t * N + n] += total[r];
   }
 }
 
@@ -195,12 +263,12 @@ extern "C" int mk_expert_down(const void* act, const void* w, int dtype, const i
                               const float* weights, float* y, int tokens, int top, int ff, int N,
                               hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && top > 0 && ff > 0 && N > 0, "expert_down: bad sizes");
-  MK_REQUIRE((size_t)top * ff * 4 <= 64 * 1024, "expert_down: %d rows of %d are too many", top, ff);
+  MK_REQUIRE((size_t)ff * 4 <= 64 * 1024, "expert_down: rows of %d are too wide", ff);
   if (tokens == 0) return 0;
   const int per_block = 4 * EXPERT_ROWS_PER_WAVE;
   dim3 grid(tokens, (N + per_block - 1) / per_block);
   MK_REQUIRE(grid.y <= 65535, "expert_down: N=%d too large for one launch", N);
-  const size_t lds = (size_t)top * ff * 4;
+  const size_t lds = (size_t)ff * 4;
   if (dtype == MK_F32)
     expert_down_kernel<float><<<grid, 256, lds, stream>>>((const float*)act, (const float*)w, ids,
                                                           weights, y, top, ff, N);

@@ -71,6 +71,9 @@ struct QkvTarget {
   bf16_t* k_cache;         // [pages, n_kv, page, d]
   bf16_t* v_cache;         // [pages, n_kv, d, page]
   int page_shift, n_q, n_kv, d, rotate;
+  // gated epilogues: the activation MK_ACT_* and its constants (all zero: SiLU)
+  int act_kind;
+  float act_limit, act_alpha, act_beta;
 };
 
 struct SkinnyArgs : QkvTarget {
@@ -97,6 +100,18 @@ extern __shared__ __align__(16) unsigned char skinny_rows[];
 // (reference: mercury/model/qwen2.py:42)
 __device__ __forceinline__ float silu_for_bf16(float g) {
   return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * -1.44269504088896340736f));
+}
+
+// The gated epilogues' value from the (bfloat16-rounded) gate and up products.  SiLU rounds
+// silu(g) before it multiplies, as the unfused kernels do; the clamped form
+// g' * sigmoid(alpha g') * (u' + beta), g' = min(g, limit), u' = clamp(u, -limit, limit), is
+// rounded once, by whoever stores it.
+__device__ __forceinline__ float gated_value(float g, float u, const QkvTarget& a) {
+  if (a.act_kind == MK_ACT_SILU) return Elem<bf16_t>::round(silu_for_bf16(g)) * u;
+  g = fminf(g, a.act_limit);
+  u = fminf(fmaxf(u, -a.act_limit), a.act_limit);
+  return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * a.act_alpha * -1.44269504088896340736f)) *
+         (u + a.act_beta);
 }
 
 __device__ __forceinline__ float load_scalar(const void* p, int is_bf16, int i) {
@@ -478,7 +493,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float g = Elem<bf16_t>::round(acc[0][tb][i]), u = Elem<bf16_t>::round(acc[1][tb][i]);
-        o[i] = f32_to_bf16(Elem<bf16_t>::round(silu_for_bf16(g)) * u);
+        o[i] = f32_to_bf16(gated_value(g, u, p));
       }
       if (n + 3 < N && (N & 3) == 0) {
         *(ushort4*)(dst + n) = make_ushort4(o[0], o[1], o[2], o[3]);
@@ -682,11 +697,23 @@ extern "C" int mk_linear_skinny_acc(const void* x, const void* w, const void* bi
 // act[M, I] = silu(x Wg^T) * (x Wu^T) for W = [Wg | Wu] stacked as [2 I, K], 1 <= M <= 16.
 extern "C" int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
                                hipStream_t stream) {
+  return mk_gated_skinny_act(x, w, act, M, inter, K, MK_ACT_SILU, 0.f, 1.f, 0.f, stream);
+}
+
+// The same with the activation MK_ACT_* `kind` and its constants in the epilogue.
+extern "C" int mk_gated_skinny_act(const void* x, const void* w, void* act, int M, int inter,
+                                   int K, int kind, float limit, float alpha, float beta,
+                                   hipStream_t stream) {
   MK_REQUIRE(M >= 1 && M <= 16, "gated projection: M=%d outside 1..16", M);
   MK_REQUIRE(inter > 0 && K > 0 && K % 8 == 0, "gated projection: K=%d must be a multiple of 8",
              K);
-  launch_skinny<2, SK_GATED>(skinny_args(x, w, act, M, inter, K, (K + 127) / 128),
-                             dim3((inter + 15) / 16, 1), stream);
+  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP, "gated projection: activation %d", kind);
+  SkinnyArgs a = skinny_args(x, w, act, M, inter, K, (K + 127) / 128);
+  a.act_kind = kind;
+  a.act_limit = limit;
+  a.act_alpha = alpha;
+  a.act_beta = beta;
+  launch_skinny<2, SK_GATED>(a, dim3((inter + 15) / 16, 1), stream);
   MK_LAUNCH_CHECK("gated_skinny");
   return 0;
 }
@@ -1141,7 +1168,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
         for (int i = 0; i < 4; ++i) {
           const float g = Elem<bf16_t>::round(acc[ta][tb][i]);
           const float u = Elem<bf16_t>::round(acc[ta][tb + TN / 2][i]);
-          o[i] = Elem<bf16_t>::round(silu_for_bf16(g)) * u;
+          o[i] = gated_value(g, u, target);
         }
         if (n + 3 < N && (ldo & 3) == 0) {
           *(uint2*)dst = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
@@ -1372,12 +1399,25 @@ extern "C" int mk_linear_tiled_partials(const void* x, const void* w, float* out
 // act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K].
 extern "C" int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K,
                               int config, hipStream_t stream) {
+  return mk_gated_tiled_act(x, w, act, M, inter, K, config, MK_ACT_SILU, 0.f, 1.f, 0.f, stream);
+}
+
+// The same with the activation MK_ACT_* `kind` and its constants in the epilogue.
+extern "C" int mk_gated_tiled_act(const void* x, const void* w, void* act, int M, int inter, int K,
+                                  int config, int kind, float limit, float alpha, float beta,
+                                  hipStream_t stream) {
+  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP, "gated projection: activation %d", kind);
+  QkvTarget target = QkvTarget();
+  target.act_kind = kind;
+  target.act_limit = limit;
+  target.act_alpha = alpha;
+  target.act_beta = beta;
   MK_REQUIRE(M > 0 && inter > 0 && K > 0 && K % 8 == 0,
              "gated projection: K=%d must be a multiple of 8 (M=%d I=%d)", K, M, inter);
   MK_REQUIRE((M + 63) / 64 <= 65535, "gated projection: M=%d too large for one launch", M);
   if (config < 0) config = tiled_config_for(M, inter, K, 2, 2);
   MK_REQUIRE(config < TILED_CONFIGS, "gated projection: no configuration %d", config);
-  launch_tiled<EPI_GATED>(config, x, w, nullptr, MK_F32, act, M, inter, K, inter, 1, stream);
+  launch_tiled<EPI_GATED>(config, x, w, nullptr, MK_F32, act, M, inter, K, inter, 1, stream, target);
   MK_LAUNCH_CHECK("gated_tiled");
   return 0;
 }

@@ -49,7 +49,8 @@ __global__ void latent_prepare_kernel(const float* __restrict__ down, int down_s
                                       const int* __restrict__ token_seq,
                                       const int* __restrict__ block_table, int table_stride,
                                       T* __restrict__ q_latent, T* __restrict__ k_cache,
-                                      T* __restrict__ v_cache, int page_shift, int write_kv) {
+                                      T* __restrict__ v_cache, int page_shift, int write_kv,
+                                      int key_width, int value_width) {
   __shared__ float scratch[16];
   extern __shared__ float rotated[];     // the token's raw rotated key part
   const int t = blockIdx.x;
@@ -72,9 +73,12 @@ __global__ void latent_prepare_kernel(const float* __restrict__ down, int down_s
   float sq = 0.f;
   for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) sq = fmaf(c[i], c[i], sq);
   const float rstd = 1.f / sqrtf(block_sum(sq, scratch) / (float)kv_rank + eps);
-  const int width = kv_rank + rot;
-  T* k_dst = k_cache + ((size_t)page * page_size + off) * width;
-  T* v_dst = v_cache + (size_t)page * kv_rank * page_size + off;
+  // rows of key_width >= kv_rank + rot and value_width >= kv_rank: what lies beyond is zero
+  T* k_dst = k_cache + ((size_t)page * page_size + off) * key_width;
+  T* v_dst = v_cache + (size_t)page * value_width * page_size + off;
+  for (int i = kv_rank + rot + threadIdx.x; i < key_width; i += blockDim.x) Elem<T>::store(k_dst + i, 0.f);
+  for (int i = kv_rank + threadIdx.x; i < value_width; i += blockDim.x)
+    Elem<T>::store(v_dst + (size_t)i * page_size, 0.f);
   for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) {
     const float v = c[i] * rstd * weight_at(kv_norm_w, norm_bf16, i);
     Elem<T>::store(k_dst + i, v);
@@ -94,8 +98,11 @@ extern "C" int mk_latent_prepare(const float* down, int down_stride, int q_rank,
                                  const float* sin_table, int table_positions, int rot_dims,
                                  int interleaved, const int* positions, const int* token_seq,
                                  const int* block_table, int table_stride, void* q_latent,
-                                 void* k_cache, void* v_cache, int dtype, int page_size,
-                                 int write_kv, int tokens, hipStream_t stream) {
+                                 void* k_cache, void* v_cache, int key_width, int value_width,
+                                 int dtype, int page_size, int write_kv, int tokens,
+                                 hipStream_t stream) {
+  MK_REQUIRE(!write_kv || (key_width >= kv_rank + rot && value_width >= kv_rank),
+             "latent_prepare: cache rows of %d / %d are too narrow", key_width, value_width);
   MK_REQUIRE(tokens >= 0 && q_rank >= 0 && kv_rank > 0 && rot >= 0, "latent_prepare: bad sizes");
   MK_REQUIRE(down_stride >= q_rank + (write_kv ? kv_rank + rot : 0),
              "latent_prepare: rows of %d hold no [%d | %d | %d]", down_stride, q_rank, kv_rank, rot);
@@ -116,7 +123,8 @@ extern "C" int mk_latent_prepare(const float* down, int down_stride, int q_rank,
   latent_prepare_kernel<T><<<tokens, threads, lds, stream>>>(                                     \
       down, down_stride, q_rank, kv_rank, rot, q_norm_w, kv_norm_w, norm_dtype == MK_BF16, eps,   \
       cos_table, sin_table, rot_dims, interleaved, positions, token_seq, block_table,             \
-      table_stride, (T*)q_latent, (T*)k_cache, (T*)v_cache, mk_log2(page_size), write_kv)
+      table_stride, (T*)q_latent, (T*)k_cache, (T*)v_cache, mk_log2(page_size), write_kv,         \
+      key_width, value_width)
   if (dtype == MK_F32) LP_LAUNCH(float);
   else if (dtype == MK_BF16) LP_LAUNCH(bf16_t);
   else MK_REQUIRE(false, "latent_prepare: unknown dtype %d", dtype);
@@ -155,6 +163,12 @@ __global__ void latent_query_tail_kernel(const T* __restrict__ q, int heads, int
     }
     Elem<T>::store(out + ((size_t)t * heads + head) * out_width + out_offset + j, y);
   }
+  // what lies behind the rotated part in a row of the output is zero
+  const int pad = out_width - out_offset - rot;
+  for (int idx = threadIdx.x; idx < heads * pad; idx += blockDim.x) {
+    const int head = idx / pad, j = idx - head * pad;
+    Elem<T>::store(out + ((size_t)t * heads + head) * out_width + out_offset + rot + j, 0.f);
+  }
 }
 
 extern "C" int mk_latent_query_tail(const void* q, int dtype, int heads, int dim, int rot,
@@ -168,8 +182,8 @@ extern "C" int mk_latent_query_tail(const void* q, int dtype, int heads, int dim
              "latent_query_tail: %d rotated dims of %d", rot_dims, rot);
   MK_REQUIRE(rot_dims == 0 || (cos_table && sin_table && table_positions > 0),
              "latent_query_tail: no angle tables");
-  if (tokens == 0 || rot == 0) return 0;
-  const int work = heads * rot;
+  if (tokens == 0 || out_offset == out_width) return 0;
+  const int work = heads * (out_width - out_offset);
   const int threads = work >= 256 ? 256 : (work + 63) / 64 * 64;
   if (dtype == MK_F32)
     latent_query_tail_kernel<float><<<tokens, threads, 0, stream>>>(

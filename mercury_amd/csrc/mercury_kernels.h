@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 22
+#define MK_ABI_VERSION 23
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
@@ -131,17 +131,20 @@ int mk_linear_batched_generic(const void* x, const void* w, int dtype, void* out
 // (the first rot_dims dims of it, pairs (2i, 2i + 1) when interleaved, else (i, i + rot_dims /
 // 2); angle tables [positions, rot_dims / 2]), written to the paged cache as one key row
 // [kv_rank + rot] of one shared head, the normed latent once more as that head's value,
-// transposed within the page ([pages, kv_rank, page_size]).  q_rank = 0: no query latent.
+// transposed within the page ([pages, value_width, page_size]).  Key rows are key_width >=
+// kv_rank + rot wide, the value has value_width >= kv_rank rows; what lies beyond is written
+// as zeros.  q_rank = 0: no query latent.
 int mk_latent_prepare(const float* down, int down_stride, int q_rank, int kv_rank, int rot,
                       const void* q_norm_w, const void* kv_norm_w, int norm_dtype, float eps,
                       const float* cos_table, const float* sin_table, int table_positions,
                       int rot_dims, int interleaved, const int* positions, const int* token_seq,
                       const int* block_table, int table_stride, void* q_latent, void* k_cache,
-                      void* v_cache, int dtype, int page_size, int write_kv, int tokens,
-                      hipStream_t stream);
+                      void* v_cache, int key_width, int value_width, int dtype, int page_size,
+                      int write_kv, int tokens, hipStream_t stream);
 
 // q [T, heads, dim + rot] -> out[t, head, out_offset .. out_offset + rot) of rows
-// [heads, out_width]: every head's rotated part, turned by the token's position.
+// [heads, out_width]: every head's rotated part, turned by the token's position, and zeros
+// behind it up to out_width.
 int mk_latent_query_tail(const void* q, int dtype, int heads, int dim, int rot,
                          const float* cos_table, const float* sin_table, int table_positions,
                          int rot_dims, int interleaved, const int* positions, void* out,
@@ -168,6 +171,15 @@ int mk_gate_act(const void* gate_up, void* out, int dtype, int tokens, int inter
 
 // h[i] += mult * (y[i] + sum_k a[k * stride + i] + sum_k b[k * stride + i]) for i < n; y may
 // be null.  mk_fill_zero: p[i] = 0 by a kernel (a captured graph records no memset node).
+// Pairs (token, choice) grouped by expert: rows [pairs] lists the pair indices expert by
+// expert (in no particular order within an expert), offsets [experts + 1] where each expert's
+// group starts.  One workgroup.  mk_expert_combine: y[t, :] += sum_j pairs_out[t * top + j, :],
+// j ascending.
+int mk_route_group(const int* ids, int pairs, int experts, int* rows, int* offsets,
+                   hipStream_t stream);
+int mk_expert_combine(const float* pairs_out, float* y, int tokens, int top, int N,
+                      hipStream_t stream);
+
 int mk_scaled_add(float* h, const float* y, const float* a, int na, const float* b, int nb,
                   long long stride, float mult, long long n, hipStream_t stream);
 int mk_fill_zero(float* p, long long n, hipStream_t stream);
@@ -195,6 +207,9 @@ int mk_linear_skinny_fixed(const void* x, const void* w, const void* bias, int b
 // 1 <= M <= 16.
 int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
                     hipStream_t stream);
+// The same with the gate activation MK_ACT_* `kind` (limit, alpha, beta: its constants).
+int mk_gated_skinny_act(const void* x, const void* w, void* act, int M, int inter, int K, int kind,
+                        float limit, float alpha, float beta, hipStream_t stream);
 
 // The gated and the q/k/v projection of at most 16 rows on x = rmsnorm(h64) * norm_w, which
 // every workgroup makes for itself from the fixed-point residual stream h64 [M, K] (the norm
@@ -231,6 +246,42 @@ int mk_qkv_tiled(const void* x, const void* w, const void* bias, int bias_dtype,
 int mk_gated_tiled_config(int M, int inter, int K);
 int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K, int config,
                    hipStream_t stream);
+int mk_gated_tiled_act(const void* x, const void* w, void* act, int M, int inter, int K, int config,
+                       int kind, float limit, float alpha, float beta, hipStream_t stream);
+
+// Many small products in one launch: y_b = x_b W_b^T for b < batch, x_b = x + b * x_batch (rows
+// lda apart), W_b = w + b * w_batch ([N, K]), y_b = out + b * o_batch (rows ldo apart), offsets
+// in elements, everything bfloat16; K, lda and the offsets multiples of 8.
+int mk_linear_batched_mfma(const void* x, const void* w, void* out, int M, int N, int K, int lda,
+                           int ldo, int batch, long long x_batch, long long w_batch,
+                           long long o_batch, hipStream_t stream);
+
+// Experts over the tokens routed to them.  rows [T * top] lists the (token, choice) pairs
+// grouped by expert, offsets [experts + 1] where each expert's group starts, max_rows bounds a
+// group's size.  gated: act[pair, :] (bfloat16 [T * top, ff]) = activation(Wg[e] x[pair / top],
+// Wu[e] x[pair / top]) for w [experts, 2 ff, K].  down: y[pair, :] (float32 [T * top, N]) =
+// weights[pair] * Wd[e] act[pair, :] for w [experts, N, ff].
+int mk_expert_gated_mfma(const void* x, const void* w, void* act, const int* rows,
+                         const int* offsets, int experts, int max_rows, int top, int ff, int K,
+                         int kind, float limit, float alpha, float beta, hipStream_t stream);
+int mk_expert_down_mfma(const void* act, const void* w, float* y, const int* rows,
+                        const int* offsets, const float* weights, int experts, int max_rows, int ff,
+                        int N, hipStream_t stream);
+
+// Attention of `heads` query heads over one shared key/value head with keys of dk (a multiple
+// of 32) and values of dv dims (a multiple of 16): q [T, heads, dk], out [T, heads, dv], keys
+// [pages, page, dk], values transposed within the page [pages, dv, page].  Tiles of 16 rows,
+// row f of a sequence = token f / heads, head f % heads (tile_seq / tile_row0 as for
+// mk_attention_mfma with one group of `heads`).  num_parts > 1 splits every tile's keys into
+// that many parts (at most mk_attention_latent_max_parts()) whose results part_o
+// [tiles, parts, dv, 16] / part_ml [tiles, parts, 2, 16] a second kernel merges.  No window.
+int mk_attention_latent_supported(int dk, int dv, int page_size);
+int mk_attention_latent_max_parts(void);
+int mk_attention_latent(const void* q, void* out, const void* k_cache, const void* v_cache,
+                        const int* tile_seq, const int* tile_row0, int num_tiles, const int* cu_q,
+                        const int* kv_len, const int* block_table, int table_stride, int page_size,
+                        int heads, int dk, int dv, float scale, int num_parts, float* part_o,
+                        float* part_ml, hipStream_t stream);
 
 // y = x W^T (+ bias) for any M, tiled through LDS; output bfloat16 or float32, or float32
 // accumulated into `out`.  config: a tile configuration, 0 .. mk_linear_tiled_configs() - 1

@@ -162,21 +162,26 @@ int run_latent_attention(const void* params, mk_op_context* ctx) {
     Launch l(ctx);
     const StepArrays arrays = arrays_of(s, p.group);
     const Queries q = latent_queries(l, ctx->x, s.num_tokens, ctx->hidden, a, arrays);
-    AttendArgs at;
-    at.n_q = a.heads;
-    at.n_kv = 1;
-    at.head_dim = a.key_width();
-    at.value_dim = a.kv_rank;
-    at.page_size = a.page_size;
-    at.window = p.window;
-    at.scale = p.scale;
-    at.k_cache = a.k_cache;
-    at.v_cache = a.v_cache;
-    const void* summed = attend(l, q, at, arrays, s);
+    if (p.window) throw KernelError("latent attention sees every earlier token: no window");
+    const void* summed = latent_attend(l, q, a, p.scale, arrays, s);
     const void* values = latent_values(l, summed, s.num_tokens, a);
     project_into_stream(l, values, s.num_tokens, p.w_o, ctx->hidden, a.heads * a.vdim, nullptr, kF32,
                         ctx->h, ctx->out_pending, ctx->out_pending_count);
   });
+}
+
+int tiles_latent_attention(const void* params, const mk_step_shape* shape, mk_tile_need* out) {
+  const LatentAttentionParams& p = *static_cast<const LatentAttentionParams*>(params);
+  mk_step_view view;
+  std::memset(&view, 0, sizeof view);
+  view.num_seqs = shape->num_seqs;
+  view.counts = shape->counts;
+  view.max_q_len = shape->max_q_len;
+  view.max_kv_len = shape->max_kv_len;
+  if (!latent_plan(shape->dtype, p.latent, view).mfma) return 0;
+  out->group = p.latent.heads;
+  out->tile_rows = 16;
+  return 1;
 }
 
 int run_routed_experts(const void* params, mk_op_context* ctx) {
@@ -267,7 +272,7 @@ void register_builtin_ops() {
   r.add(OpKind{"norm", &run_norm, nullptr, MK_OP_FOLDS_PENDING | MK_OP_FIXED_STREAM});
   r.add(OpKind{"attention", &run_attention, &tiles_attention, MK_OP_READS_X | MK_OP_FIXED_STREAM});
   r.add(OpKind{"gated_mlp", &run_gated_mlp, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
-  r.add(OpKind{"latent_attention", &run_latent_attention, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"latent_attention", &run_latent_attention, &tiles_latent_attention, MK_OP_READS_X});
   r.add(OpKind{"routed_experts", &run_routed_experts, nullptr, MK_OP_READS_X});
   r.add(OpKind{"parallel", &run_parallel, &tiles_parallel, MK_OP_READS_X});
   r.add(OpKind{"head", &run_head, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});

@@ -1,6 +1,8 @@
 #include "launch.h"
 
+#include <algorithm>
 #include <string>
+#include <vector>
 
 #include "kernels.h"
 
@@ -372,27 +374,30 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
 
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
             int tile_config, const NormFold* fold, const GateAct& act) {
-  const bool fuses = act.silu() && fuses_gating(l.dtype(), l.dtype(), m, k, 2 * inter);
-  const bool folded = fold && fuses && tile_config == -2 && m <= 16 && folds_norm(l.dtype(), m, k);
+  const bool fuses = fuses_gating(l.dtype(), l.dtype(), m, k, 2 * inter);
+  const bool folded = fold && fuses && act.silu() && tile_config == -2 && m <= 16 &&
+                      folds_norm(l.dtype(), m, k);
   if (fold && !folded) {
     x = rmsnorm_fixed(l, fold->h64, k, fold->weight, fold->weight_dtype, fold->eps, nullptr, m);
   }
   if (fuses) {
-    void* act = l.alloc((size_t)m * inter * 2);
-    if (l.dry() || m == 0) return act;
+    void* out = l.alloc((size_t)m * inter * 2);
+    if (l.dry() || m == 0) return out;
     const KernelTable& t = need_mfma();
     if (folded) {
       check_mfma(t.mk_gated_skinny_normed(fold->h64, fold->weight, fold->weight_dtype, fold->eps,
-                                          w_gate_up, act, m, inter, k, l.stream()),
+                                          w_gate_up, out, m, inter, k, l.stream()),
                  "gated_projection");
-      return act;
+      return out;
     }
     const bool skinny = gated_is_skinny(m) && tile_config == -2;
-    check_mfma(skinny ? t.mk_gated_skinny(x, w_gate_up, act, m, inter, k, l.stream())
-                      : t.mk_gated_tiled(x, w_gate_up, act, m, inter, k,
-                                         tile_config == -2 ? -1 : tile_config, l.stream()),
+    check_mfma(skinny ? t.mk_gated_skinny_act(x, w_gate_up, out, m, inter, k, act.kind, act.limit,
+                                              act.alpha, act.beta, l.stream())
+                      : t.mk_gated_tiled_act(x, w_gate_up, out, m, inter, k,
+                                             tile_config == -2 ? -1 : tile_config, act.kind,
+                                             act.limit, act.alpha, act.beta, l.stream()),
                "gated_projection");
-    return act;
+    return out;
   }
   if (tile_config != -2) throw KernelError("gated_projection: operands not eligible");
   void* gate_up = linear(l, x, m, w_gate_up, 2 * inter, k, nullptr, kF32, nullptr, l.dtype(), false);
@@ -407,6 +412,15 @@ void* linear_per_head(Launch& l, const void* x, int m, int heads, int lda, int x
     o_head = n;
   }
   if (l.dry() || m == 0) return out;
+  // the matrix-core kernel wants 16-byte pieces of rows: K, the row pitch and the heads' offsets
+  // multiples of 8 elements
+  if (l.dtype() == kBF16 && kernels().has_mfma() && k % 8 == 0 && lda % 8 == 0 && x_head % 8 == 0 &&
+      ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
+    check_mfma(need_mfma().mk_linear_batched_mfma(x, w, out, m, n, k, lda, ldo, heads, x_head,
+                                                  (long long)n * k, o_head, l.stream()),
+               "linear_per_head");
+    return out;
+  }
   check_core(need_core().mk_linear_batched_generic(x, w, l.dtype(), out, l.dtype(), m, n, k, lda,
                                                    ldo, heads, x_head, (long long)n * k, o_head,
                                                    l.stream()), "linear_per_head");
@@ -426,8 +440,9 @@ Queries latent_queries(Launch& l, const void* x, int m, int hidden, const Latent
                    down, down_width, a.q_rank, a.kv_rank, a.rot, a.q_norm, a.kv_norm, a.norm_dtype,
                    a.eps, a.pos.cos, a.pos.sin, a.pos.table_positions, a.pos.rotary_dim,
                    a.pos.interleaved, s.positions, s.token_seq, s.table, s.table_stride, q_latent,
-                   a.writes ? a.k_cache : nullptr, a.writes ? a.v_cache : nullptr, l.dtype(),
-                   a.writes ? a.page_size : 1, a.writes ? 1 : 0, m, l.stream()), "latent_prepare");
+                   a.writes ? a.k_cache : nullptr, a.writes ? a.v_cache : nullptr, a.key_width(),
+                   a.value_width(), l.dtype(), a.writes ? a.page_size : 1, a.writes ? 1 : 0, m,
+                   l.stream()), "latent_prepare");
   }
   const void* q = linear(l, q_latent, m, a.w_uq, a.heads * per_head, a.q_rank, nullptr, kF32,
                          nullptr, l.dtype(), false);
@@ -443,9 +458,61 @@ Queries latent_queries(Launch& l, const void* x, int m, int hidden, const Latent
   return {out, a.heads * width};
 }
 
+namespace {
+// Decoding with few tiles: the keys are cut into parts until about this many wavefronts run,
+// a part being at least this many blocks of 32 keys.
+constexpr int kLatentWaves = 1024;
+constexpr int kLatentMinBlocks = 4;
+}  // namespace
+
+LatentPlan latent_plan(int dtype, const LatentArgs& a, const mk_step_view& step) {
+  LatentPlan plan;
+  if (dtype != kBF16 || !kernels().has_mfma()) return plan;
+  const KernelTable& t = need_mfma();
+  if (!t.mk_attention_latent_supported(a.key_width(), a.value_width(), a.page_size)) return plan;
+  plan.mfma = true;
+  const std::vector<int> counts(step.counts, step.counts + step.num_seqs);
+  plan.num_tiles = count_tiles(counts, a.heads, 16);
+  const int blocks = (step.max_kv_len + 31) / 32;
+  int parts = 1;
+  if (plan.num_tiles > 0 && plan.num_tiles < kLatentWaves) {
+    parts = std::min(kLatentWaves / plan.num_tiles, std::max(1, blocks / kLatentMinBlocks));
+  }
+  plan.parts = std::max(1, std::min(parts, t.mk_attention_latent_max_parts()));
+  return plan;
+}
+
+void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scale,
+                    const StepArrays& s, const mk_step_view& step) {
+  const int m = step.num_tokens, dk = a.key_width(), dv = a.value_width();
+  void* out = l.alloc((size_t)m * a.heads * dv * l.elem());
+  const LatentPlan plan = latent_plan(l.dtype(), a, step);
+  if (!plan.mfma) {
+    if (!l.dry() && m > 0) {
+      check_core(need_core().mk_attention_generic_kv(
+                     q.q, q.stride, out, a.heads * dv, a.k_cache, a.v_cache, l.dtype(), s.positions,
+                     s.token_seq, s.table, s.table_stride, a.page_size, a.heads, 1, dk, dv, scale,
+                     0, 0.f, nullptr, m, l.stream()), "latent_attention");
+    }
+    return out;
+  }
+  float *part_o = nullptr, *part_ml = nullptr;
+  if (plan.parts > 1) {
+    part_o = (float*)l.alloc((size_t)plan.num_tiles * plan.parts * dv * 16 * 4);
+    part_ml = (float*)l.alloc((size_t)plan.num_tiles * plan.parts * 32 * 4);
+  }
+  if (l.dry() || m == 0) return out;
+  const mk_tile_list& tiles = tiles_for(step, a.heads, 16);
+  check_mfma(need_mfma().mk_attention_latent(q.q, out, a.k_cache, a.v_cache, tiles.seq, tiles.row0,
+                                             tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride,
+                                             a.page_size, a.heads, dk, dv, scale, plan.parts, part_o,
+                                             part_ml, l.stream()), "latent_attention");
+  return out;
+}
+
 void* latent_values(Launch& l, const void* summed, int m, const LatentArgs& a) {
-  return linear_per_head(l, summed, m, a.heads, a.heads * a.kv_rank, a.kv_rank, a.w_uv, a.vdim,
-                         a.kv_rank, nullptr, 0, 0);
+  return linear_per_head(l, summed, m, a.heads, a.heads * a.value_width(), a.value_width(), a.w_uv,
+                         a.vdim, a.kv_rank, nullptr, 0, 0);
 }
 
 void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y) {
@@ -454,10 +521,33 @@ void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArg
   int* ids = (int*)l.alloc((size_t)m * a.top * 4);
   float* weights = (float*)l.alloc((size_t)m * a.top * 4);
   void* act = l.alloc((size_t)m * a.top * a.ff * l.elem());
+  // On the matrix cores the (token, choice) pairs are grouped by expert, so that an expert's
+  // matrices are multiplied with all its tokens at once; every pair's down-projection lands in
+  // a row of its own and the rows of a token are added in the order of its choices.
+  const bool grouped = l.dtype() == kBF16 && kernels().has_mfma() && hidden % 8 == 0 &&
+                       a.ff % 8 == 0 && a.experts <= 1024;
+  int *rows = nullptr, *offsets = nullptr;
+  float* pair_out = nullptr;
+  if (grouped) {
+    rows = (int*)l.alloc((size_t)m * a.top * 4);
+    offsets = (int*)l.alloc((size_t)(a.experts + 1) * 4);
+    pair_out = (float*)l.alloc((size_t)m * a.top * hidden * 4);
+  }
   if (l.dry() || m == 0) return;
   const KernelTable& t = need_core();
   check_core(t.mk_route_topk(logits, a.experts, a.top, a.scale, a.renormalize, ids, weights, m,
                              l.stream()), "route");
+  if (grouped) {
+    const KernelTable& f = need_mfma();
+    check_core(t.mk_route_group(ids, m * a.top, a.experts, rows, offsets, l.stream()), "route_group");
+    check_mfma(f.mk_expert_gated_mfma(x, a.w_gate_up, act, rows, offsets, a.experts, m, a.top, a.ff,
+                                      hidden, a.act.kind, a.act.limit, a.act.alpha, a.act.beta,
+                                      l.stream()), "expert_gated");
+    check_mfma(f.mk_expert_down_mfma(act, a.w_down, pair_out, rows, offsets, weights, a.experts, m,
+                                     a.ff, hidden, l.stream()), "expert_down");
+    check_core(t.mk_expert_combine(pair_out, y, m, a.top, hidden, l.stream()), "expert_combine");
+    return;
+  }
   check_core(t.mk_expert_gated(x, a.w_gate_up, l.dtype(), ids, act, m, a.top, a.ff, hidden,
                                a.act.kind, a.act.limit, a.act.alpha, a.act.beta, l.stream()),
              "expert_gated");

@@ -214,13 +214,23 @@ struct LatentArgs {
   void *k_cache = nullptr, *v_cache = nullptr;
   int page_size = 1;
   bool writes = true;
-  int key_width() const { return kv_rank + rot; }
+  // rows as the cache holds them: padded to what the matrix-core attention takes
+  int key_width() const { return (kv_rank + rot + 31) / 32 * 32; }
+  int value_width() const { return (kv_rank + 15) / 16 * 16; }
 };
 // Down-projection, norms, rotation and cache write, query up-projection; the queries come back
 // as rows [heads, kv_rank + rot] = [absorbed | rotated].
 Queries latent_queries(Launch& l, const void* x, int m, int hidden, const LatentArgs& a,
                        const StepArrays& s);
-// [m, heads, kv_rank] weighted sums of latents -> [m, heads vdim] values.
+// The attention over the cached latents: [m, heads, value_width()] weighted sums of them.
+struct LatentPlan {
+  bool mfma = false;
+  int parts = 1, num_tiles = 0;
+};
+LatentPlan latent_plan(int dtype, const LatentArgs& a, const mk_step_view& step);
+void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scale,
+                    const StepArrays& s, const mk_step_view& step);
+// [m, heads, value_width()] weighted sums of latents -> [m, heads vdim] values.
 void* latent_values(Launch& l, const void* summed, int m, const LatentArgs& a);
 
 // Routed experts: router logits in float32, the `top` of softmax, and

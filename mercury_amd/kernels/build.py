@@ -40,7 +40,9 @@ LIBRARIES = {
         "host_support.hip",
         "attention_mfma.hip",
         "attention_out.hip",
+        "attention_latent.hip",
         "gemm_mfma.hip",
+        "gemm_batched_mfma.hip",
     ],
 }
 

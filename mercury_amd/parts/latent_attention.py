@@ -57,7 +57,11 @@ class LatentAttention(Mixer):
         self._alone: dict = {}
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(1, self.kv_rank + self.rot_dim, self.window, value_dim=self.kv_rank)
+        # one shared head; rows padded to what the matrix-core attention takes (key rows to a
+        # multiple of 32, the transposed values to a multiple of 16), the padding zero
+        key_width = -(-(self.kv_rank + self.rot_dim) // 32) * 32
+        value_width = -(-self.kv_rank // 16) * 16
+        return CacheSpec(1, key_width, self.window, value_dim=value_width)
 
     def param_specs(self) -> dict:
         n, per_head = self.names, self.dim + self.rot_dim
