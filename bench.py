@@ -18,6 +18,13 @@ the same run: a streaming read of a 2 GiB matrix by the engine's one-row project
 
 times the prompt attention kernel alone at the models' head shapes, and
 
+    python bench.py --talolorn [--talolorn-only NAME]
+
+times prompts of 2,048 tokens and decode steps (batch 8, context 4,096) of the Talolorn design
+(latent attention, parallel blocks; once with dense feed-forwards, once with routed experts)
+at two sets of layer sizes, beside a Qwen2 model of the same width, depth, heads and
+feed-forward size, and
+
     python bench.py --shape 32b --serve
 
 runs a whole workload through the scheduler instead (64 requests with prompts of 2,048 tokens,
@@ -86,6 +93,11 @@ def parse_args(argv=None):
     p.add_argument("--attention", action="store_true",
                    help="instead of the engine's steps: the prompt attention kernel alone at the "
                         "head shapes of the three models, a table of times and PFLOP/s")
+    p.add_argument("--talolorn", action="store_true",
+                   help="instead of the default workload: prefill and decode throughput of the "
+                        "Talolorn design at two sets of layer sizes, beside a Qwen2 model of equal size")
+    p.add_argument("--talolorn-only", default=None,
+                   help="run one entry of the comparison only (e.g. small/talolorn-moe), for a profiler")
     p.add_argument("--serve-requests", type=int, default=64)
     p.add_argument("--serve-chunk", type=int, default=512)
     return p.parse_args(argv)
@@ -130,7 +142,8 @@ class Bench:
               f"{pages} pages", file=sys.stderr, flush=True)
 
     def tokens(self, count: int) -> list:
-        return self.torch.randint(0, self.cfg["vocab_size"], (count,), generator=self.rng).tolist()
+        vocab = self.cfg["vocab_size"] if "vocab_size" in self.cfg else self.cfg["vocab"]
+        return self.torch.randint(0, vocab, (count,), generator=self.rng).tolist()
 
     def sync(self):
         self.torch.cuda.synchronize()
@@ -377,6 +390,71 @@ def attention_main(args) -> int:
     return 0
 
 
+# Layer sizes for `--talolorn`: widths, heads and ranks of the order a served model of this kind
+# has; four layers each (the first dense), so that a run takes seconds.
+TALOLORN_SIZES = {
+    "small": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, q_rank=768, kv_rank=512,
+                  ff=8192, experts=64, top=6, expert_ff=1408, vocab=32000, layers=4),
+    "large": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, q_rank=1536, kv_rank=512,
+                  ff=12288, experts=64, top=6, expert_ff=1536, vocab=32000, layers=4),
+}
+
+
+def talolorn_configs(z: dict) -> dict:
+    """name -> config.json of the three models compared at the sizes `z`."""
+    mixer = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["vdim"],
+             "q_rank": z["q_rank"], "kv_rank": z["kv_rank"], "scale": (z["dim"] + z["rot_dim"]) ** -0.5,
+             "rot": {"base": 10000.0, "dims": z["rot_dim"]}}
+    dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "top": z["top"], "scale": 1.0}}
+    layer = lambda mlp: {"type": "latent_attention", "mixer": mixer, "mlp": mlp}
+    base = {"architecture": "Talolorn", "vocab": z["vocab"], "width": z["width"],
+            "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "residual_mult": 1.0}
+    return {
+        "talolorn-dense": dict(base, layers=[layer(dense)] * z["layers"]),
+        "talolorn-moe": dict(base, layers=[layer(dense)] + [layer(moe)] * (z["layers"] - 1)),
+        "qwen2": {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+                  "hidden_size": z["width"], "intermediate_size": z["ff"],
+                  "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+                  "num_key_value_heads": z["heads"] // 4, "head_dim": z["dim"],
+                  "vocab_size": z["vocab"], "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
+                  "tie_word_embeddings": False, "max_position_embeddings": 32768},
+    }
+
+
+def talolorn_main(args) -> int:
+    import torch
+
+    rows = {}
+    for size, z in TALOLORN_SIZES.items():
+        for name, cfg in talolorn_configs(z).items():
+            key = f"{size}/{name}"
+            if args.talolorn_only and args.talolorn_only != key:
+                continue
+            bench = Bench(cfg, args.dtype, args.batch, args.context, args.seed, not args.no_lookahead)
+            run = bench.decode(args.batch, args.context, args.steps, args.warmup)
+            pre = bench.prefill(PREFILL_TOKENS, repeats=5)
+            rows[key] = {
+                "decode_ms": round(run["ms"], 4), "decode_tok_s": round(run["tok_s"], 1),
+                "decode_read_gbs": round(run["bytes"] / (run["ms"] * 1e-3) / 1e9, 1),
+                "prefill_ms": round(pre["ms"], 3), "prefill_tok_s": round(pre["tok_s"], 1),
+                "weights_gb_a_step": round(bench.model.decode_weight_bytes() / 1e9, 3),
+                "cache_bytes_a_token": bench.runner.kv_bytes_per_token(),
+            }
+            print(f"[bench] {key}: decode b{args.batch} {run['ms']:.3f} ms/step, prefill "
+                  f"{PREFILL_TOKENS} {pre['ms']:.2f} ms", file=sys.stderr, flush=True)
+            del bench
+            torch.cuda.empty_cache()
+    print(json.dumps({
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context}, and tok/s of a "
+                  f"{PREFILL_TOKENS}-token prompt: Talolorn beside Qwen2 at equal sizes",
+        "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "sizes": TALOLORN_SIZES, "rows": rows}))
+    return 0
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     if args.gpus != 1:
@@ -385,6 +463,8 @@ def main(argv=None) -> int:
         return 2
     if args.attention:
         return attention_main(args)
+    if args.talolorn:
+        return talolorn_main(args)
     model_name, shape = SHAPES[args.shape]
     cfg = dict(shape)
     full_layers = cfg["num_hidden_layers"]
