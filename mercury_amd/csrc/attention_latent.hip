@@ -14,12 +14,12 @@
 //   O^T[dim, row] += V^T[dim, key] P^T[key, row]  A = V^T, B = P^T
 //
 // The first product leaves a lane with the probabilities the second wants from it as B.
-// Widths are multiples of 32 (keys) and 16 (values): the cache rows and the queries are
-// padded with zeros by whoever writes them.  The counts of 32-wide key chunks and 16-wide
-// value tiles are run-time numbers below a compile-time bound (MAXC, MAXT), which sizes the
-// register arrays; four bounds are compiled.  With the keys split into parts, every part
-// leaves an unnormalised result with its running maximum and sum, and a second kernel merges
-// the parts in order.
+// Widths are multiples of 32 (keys) and 16 (values) from a list of compiled shapes; the cache
+// rows and the queries are padded with zeros up to the shape by whoever writes them, so every
+// loop over a width has compile-time bounds and all loads of a block of keys are asked for
+// before its first product.  With the keys split into parts, every part leaves an
+// unnormalised result with its running maximum and sum, and a second kernel merges the parts
+// in order.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -33,12 +33,12 @@ union LFrag {
 };
 
 struct LatentAttnParams {
-  const bf16_t* q;       // [T, heads, dkc * 32]
-  bf16_t* out;           // [T, heads * dv]
-  float* part_o;         // [tile, part, dvt * 16, 16]
+  const bf16_t* q;       // [T, heads, DKC * 32]
+  bf16_t* out;           // [T, heads, DVT * 16]
+  float* part_o;         // [tile, part, DVT * 16, 16]
   float* part_ml;        // [tile, part, 2, 16]
-  const bf16_t* k_cache; // [pages, page, dkc * 32]
-  const bf16_t* v_cache; // [pages, dvt * 16, page]
+  const bf16_t* k_cache; // [pages, page, DKC * 32]
+  const bf16_t* v_cache; // [pages, DVT * 16, page]
   const int* tile_seq;
   const int* tile_row0;
   const int* cu_q;
@@ -47,18 +47,26 @@ struct LatentAttnParams {
   int table_stride;
   int page_shift;
   int heads;
-  int dkc, dvt, dv;
   float scale_log2;      // scale * log2(e)
   int num_tiles;
   int num_parts;
+  int dvt;               // for the merge kernel
 };
 
 #define LAT_WAVES 4
 
-template <int MAXC, int MAXT>
-__global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnParams p) {
+// The shapes that are compiled: (32-wide key chunks, 16-wide value tiles).  A cache is laid
+// out for the first of them that holds its widths (mk_attention_latent_widths).
+#define LATENT_SHAPES(X) \
+  X(2, 2) X(2, 4) X(3, 4) X(4, 4) X(4, 8) X(5, 8) X(6, 8) X(8, 16) X(10, 16) X(12, 16) X(18, 32) X(20, 32)
+
+// The wavefronts of a workgroup are independent (tile, part) units; the block size is a
+// launch parameter (one wavefront a workgroup when there are few units, so that they spread
+// over the compute units).
+template <int DKC, int DVT>
+__global__ __launch_bounds__(256) void attn_latent_kernel(LatentAttnParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int unit = blockIdx.x * LAT_WAVES + wave;
+  const int unit = blockIdx.x * (blockDim.x >> 6) + wave;
   if (unit >= p.num_tiles * p.num_parts) return;   // a whole wavefront; nothing is shared
   // Tiles from the last: under a causal mask the later tiles of a prompt read the most keys.
   const int tile = p.num_tiles - 1 - unit / p.num_parts;
@@ -79,19 +87,18 @@ __global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnP
   const int per = (blocks + p.num_parts - 1) / p.num_parts;
   const int b_begin = part * per, b_end = min(blocks, b_begin + per);
   const int ps = 1 << p.page_shift;
-  const int dkp = p.dkc * 32, dvp = p.dvt * 16;
+  constexpr int DK = DKC * 32, DV = DVT * 16;
   const int* table = p.block_table + (size_t)seq * p.table_stride;
 
-  LFrag qf[MAXC];
+  LFrag qf[DKC];
   {
-    const bf16_t* qrow = p.q + ((size_t)token * p.heads + head) * dkp + g4 * 8;
+    const bf16_t* qrow = p.q + ((size_t)token * p.heads + head) * DK + g4 * 8;
 #pragma unroll
-    for (int c = 0; c < MAXC; ++c)
-      if (c < p.dkc) qf[c].u = *(const uint4*)(qrow + c * 32);
+    for (int c = 0; c < DKC; ++c) qf[c].u = *(const uint4*)(qrow + c * 32);
   }
-  f32x4 acc[MAXT];
+  f32x4 acc[DVT];
 #pragma unroll
-  for (int t = 0; t < MAXT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < DVT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, lsum = 0.f;
   const float c2 = p.scale_log2;
 
@@ -106,23 +113,53 @@ __global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnP
       // a half past the sequence's pages reads page 0, which exists; its keys are masked
       const int page = index < p.table_stride ? max(table[index], 0) : 0;
       const int off = kh & (ps - 1);
-      kbase[h] = p.k_cache + ((size_t)page * ps + off + r) * dkp + g4 * 8;
-      vbase[h] = p.v_cache + ((size_t)page * dvp + r) * ps + off + g4 * 4;
+      kbase[h] = p.k_cache + ((size_t)page * ps + off + r) * DK + g4 * 8;
+      vbase[h] = p.v_cache + ((size_t)page * DV + r) * ps + off + g4 * 4;
     }
+    // Everything the block needs is asked for before the first product where the registers
+    // hold it all; the widest shapes take the keys half by half and the values after them.
+    constexpr bool EARLY = DKC * 12 + DVT * 8 <= 320;
+    LFrag vf[DVT];
     float s[8];
+    if constexpr (EARLY) {
+      LFrag kf[2][DKC];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int c = 0; c < MAXC; ++c) {
-        if (c < p.dkc) {
-          LFrag kf;
-          kf.u = *(const uint4*)(kbase[h] + c * 32);
-          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sc, 0, 0, 0);
-        }
+        for (int c = 0; c < DKC; ++c) kf[h][c].u = *(const uint4*)(kbase[h] + c * 32);
+#pragma unroll
+      for (int t = 0; t < DVT; ++t) {
+        vf[t].u2[0] = *(const uint2*)(vbase[0] + (size_t)t * 16 * ps);
+        vf[t].u2[1] = *(const uint2*)(vbase[1] + (size_t)t * 16 * ps);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) s[h * 4 + i] = sc[i];
+      for (int h = 0; h < 2; ++h) {
+        f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < DKC; ++c)
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[h][c].v, qf[c].v, sc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[h * 4 + i] = sc[i];
+      }
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        LFrag kf[DKC];
+#pragma unroll
+        for (int c = 0; c < DKC; ++c) kf[c].u = *(const uint4*)(kbase[h] + c * 32);
+        f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < DKC; ++c)
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c].v, qf[c].v, sc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[h * 4 + i] = sc[i];
+        __builtin_amdgcn_sched_barrier(0);   // the next loads stay behind these products
+      }
+#pragma unroll
+      for (int t = 0; t < DVT; ++t) {
+        vf[t].u2[0] = *(const uint2*)(vbase[0] + (size_t)t * 16 * ps);
+        vf[t].u2[1] = *(const uint2*)(vbase[1] + (size_t)t * 16 * ps);
+      }
     }
     if (key0 + 31 > all_see) {   // the block holds keys some row does not see
 #pragma unroll
@@ -140,7 +177,7 @@ __global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnP
       const float corr = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
       lsum *= corr;
 #pragma unroll
-      for (int t = 0; t < MAXT; ++t) acc[t] *= corr;
+      for (int t = 0; t < DVT; ++t) acc[t] *= corr;
       m = m_new;
     }
     const float m_use = m == -INFINITY ? 0.f : m;
@@ -152,14 +189,8 @@ __global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnP
     pf.u = make_uint4(pack_bf16x2(e[0], e[1]), pack_bf16x2(e[2], e[3]), pack_bf16x2(e[4], e[5]),
                       pack_bf16x2(e[6], e[7]));
 #pragma unroll
-    for (int t = 0; t < MAXT; ++t) {
-      if (t < p.dvt) {
-        LFrag vf;
-        vf.u2[0] = *(const uint2*)(vbase[0] + (size_t)t * 16 * ps);
-        vf.u2[1] = *(const uint2*)(vbase[1] + (size_t)t * 16 * ps);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
-      }
-    }
+    for (int t = 0; t < DVT; ++t)
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pf.v, acc[t], 0, 0, 0);
   }
   // a row's sum lies in its four lanes
   lsum += __shfl_xor(lsum, 16, 64);
@@ -168,27 +199,19 @@ __global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnP
   if (p.num_parts == 1) {
     if (!row_ok) return;
     const float inv = 1.f / lsum;
-    bf16_t* dst = p.out + ((size_t)token * p.heads + head) * p.dv;
+    bf16_t* dst = p.out + ((size_t)token * p.heads + head) * DV + g4 * 4;
 #pragma unroll
-    for (int t = 0; t < MAXT; ++t) {
-      if (t < p.dvt) {
-        const int d = t * 16 + g4 * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (d + i < p.dv) dst[d + i] = f32_to_bf16(acc[t][i] * inv);
-      }
-    }
+    for (int t = 0; t < DVT; ++t)
+      *(uint2*)(dst + t * 16) = make_uint2(pack_bf16x2(acc[t][0] * inv, acc[t][1] * inv),
+                                           pack_bf16x2(acc[t][2] * inv, acc[t][3] * inv));
     return;
   }
   // [tile, part, dim, row]: a lane's four dims of its row
-  float* po = p.part_o + ((size_t)tile * p.num_parts + part) * dvp * 16;
+  float* po = p.part_o + ((size_t)tile * p.num_parts + part) * DV * 16;
 #pragma unroll
-  for (int t = 0; t < MAXT; ++t) {
-    if (t < p.dvt) {
+  for (int t = 0; t < DVT; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) po[(size_t)(t * 16 + g4 * 4 + i) * 16 + r] = acc[t][i];
-    }
-  }
+    for (int i = 0; i < 4; ++i) po[(size_t)(t * 16 + g4 * 4 + i) * 16 + r] = acc[t][i];
   if (g4 == 0) {
     float* ml = p.part_ml + ((size_t)tile * p.num_parts + part) * 32;
     ml[r] = m;
@@ -196,15 +219,18 @@ __global__ __launch_bounds__(64 * LAT_WAVES) void attn_latent_kernel(LatentAttnP
   }
 }
 
-// One workgroup per tile: the parts' results added up in part order.
+#define LATENT_MAX_PARTS 64
+
+// grid (tiles, value tiles / 4): a workgroup adds up the parts' results of 64 dims of a tile's
+// rows, in part order.
 __global__ __launch_bounds__(256) void attn_latent_merge_kernel(LatentAttnParams p) {
-  __shared__ float weight[64][16];   // at most 64 parts
+  __shared__ float weight[LATENT_MAX_PARTS][16];
   __shared__ float inv[16];
   const int tile = blockIdx.x;
   const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
   const int rows = q_len * p.heads;
-  const int dvp = p.dvt * 16;
+  const int dv = p.dvt * 16;
   const float* ml = p.part_ml + (size_t)tile * p.num_parts * 32;
   if (threadIdx.x < 16) {
     const int r = threadIdx.x;
@@ -220,24 +246,42 @@ __global__ __launch_bounds__(256) void attn_latent_merge_kernel(LatentAttnParams
     inv[r] = 1.f / total;
   }
   __syncthreads();
-  const float* po = p.part_o + (size_t)tile * p.num_parts * dvp * 16;
-  for (int idx = threadIdx.x; idx < dvp * 16; idx += blockDim.x) {
+  const float* po = p.part_o + (size_t)tile * p.num_parts * dv * 16;
+  // 64 dims x 16 rows = 1024 values, four a thread
+  for (int idx = blockIdx.y * 1024 + threadIdx.x; idx < min(dv * 16, (int)(blockIdx.y + 1) * 1024);
+       idx += 256) {
     const int d = idx >> 4, r = idx & 15;
-    if (row0 + r >= rows || d >= p.dv) continue;
+    if (row0 + r >= rows) continue;
     float total = 0.f;
-    for (int s = 0; s < p.num_parts; ++s) total += weight[s][r] * po[(size_t)s * dvp * 16 + idx];
+    for (int s = 0; s < p.num_parts; ++s) total += weight[s][r] * po[(size_t)s * dv * 16 + idx];
     const int f = row0 + r;
-    p.out[((size_t)(q0 + f / p.heads) * p.heads + f % p.heads) * p.dv + d] =
-        f32_to_bf16(total * inv[r]);
+    p.out[((size_t)(q0 + f / p.heads) * p.heads + f % p.heads) * dv + d] = f32_to_bf16(total * inv[r]);
   }
 }
 
-extern "C" int mk_attention_latent_supported(int dk, int dv, int page_size) {
-  return dk > 0 && dv > 0 && dk % 32 == 0 && dv <= dk && (dv + 15) / 16 <= 32 && dk / 32 <= 18 &&
-         page_size >= 16 && mk_is_pow2(page_size);
+// The widths a cache must have for keys of at least `dk` and values of at least `dv` dims:
+// the first compiled shape that holds them; 0 when none does.
+extern "C" int mk_attention_latent_widths(int dk, int dv, int* key_width, int* value_width) {
+#define LATENT_FITS(C, T)                                 \
+  if (dk <= (C) * 32 && dv <= (T) * 16) {                 \
+    if (key_width) *key_width = (C) * 32;                 \
+    if (value_width) *value_width = (T) * 16;             \
+    return 1;                                             \
+  }
+  LATENT_SHAPES(LATENT_FITS)
+#undef LATENT_FITS
+  return 0;
 }
 
-extern "C" int mk_attention_latent_max_parts(void) { return 64; }
+extern "C" int mk_attention_latent_supported(int dk, int dv, int page_size) {
+  if (page_size < 16 || !mk_is_pow2(page_size)) return 0;
+#define LATENT_IS(C, T) if (dk == (C) * 32 && dv == (T) * 16) return 1;
+  LATENT_SHAPES(LATENT_IS)
+#undef LATENT_IS
+  return 0;
+}
+
+extern "C" int mk_attention_latent_max_parts(void) { return LATENT_MAX_PARTS; }
 
 extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache,
                                    const void* v_cache, const int* tile_seq, const int* tile_row0,
@@ -249,10 +293,11 @@ extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache
              "latent attention: keys of %d, values of %d, pages of %d are not taken", dk, dv,
              page_size);
   MK_REQUIRE(heads > 0 && num_tiles >= 0 && table_stride > 0, "latent attention: bad sizes");
-  MK_REQUIRE(num_parts >= 1 && num_parts <= 64, "latent attention: %d parts", num_parts);
+  MK_REQUIRE(num_parts >= 1 && num_parts <= LATENT_MAX_PARTS, "latent attention: %d parts", num_parts);
   MK_REQUIRE(num_parts == 1 || (part_o && part_ml), "latent attention: parts without a workspace");
   MK_REQUIRE(q && out && k_cache && v_cache && tile_seq && tile_row0 && cu_q && kv_len && block_table,
              "latent attention: null argument");
+  MK_REQUIRE(scale > 0.f, "latent attention: the scale must be positive");
   if (num_tiles == 0) return 0;
   LatentAttnParams p;
   p.q = (const bf16_t*)q;
@@ -269,22 +314,23 @@ extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache
   p.table_stride = table_stride;
   p.page_shift = mk_log2(page_size);
   p.heads = heads;
-  p.dkc = dk / 32;
-  p.dvt = (dv + 15) / 16;
-  p.dv = dv;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.num_tiles = num_tiles;
   p.num_parts = num_parts;
+  p.dvt = dv / 16;
   const long long units = (long long)num_tiles * num_parts;
-  MK_REQUIRE((units + LAT_WAVES - 1) / LAT_WAVES < (1ll << 31), "latent attention: too many tiles");
-  const dim3 grid((unsigned)((units + LAT_WAVES - 1) / LAT_WAVES));
-  if (p.dkc <= 3 && p.dvt <= 4) attn_latent_kernel<3, 4><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
-  else if (p.dkc <= 6 && p.dvt <= 8) attn_latent_kernel<6, 8><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
-  else if (p.dkc <= 10 && p.dvt <= 16) attn_latent_kernel<10, 16><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
-  else attn_latent_kernel<18, 32><<<grid, 64 * LAT_WAVES, 0, stream>>>(p);
+  // few units: one wavefront a workgroup, so that they spread over the compute units
+  const int waves = units >= 2048 ? LAT_WAVES : 1;
+  MK_REQUIRE((units + waves - 1) / waves < (1ll << 31), "latent attention: too many tiles");
+  const dim3 grid((unsigned)((units + waves - 1) / waves));
+#define LATENT_LAUNCH(C, T)                                                   \
+  if (dk == (C) * 32 && dv == (T) * 16)                                       \
+    attn_latent_kernel<C, T><<<grid, 64 * waves, 0, stream>>>(p);
+  LATENT_SHAPES(LATENT_LAUNCH)
+#undef LATENT_LAUNCH
   MK_LAUNCH_CHECK("attention_latent");
   if (num_parts > 1) {
-    attn_latent_merge_kernel<<<num_tiles, 256, 0, stream>>>(p);
+    attn_latent_merge_kernel<<<dim3(num_tiles, (p.dvt + 3) / 4), 256, 0, stream>>>(p);
     MK_LAUNCH_CHECK("attention_latent_merge");
   }
   return 0;

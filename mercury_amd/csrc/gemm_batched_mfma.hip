@@ -52,8 +52,10 @@ __device__ __forceinline__ float batched_act(float g, float u, const BatchedPara
   return g / (1.f + __expf(-p.alpha * g)) * (u + p.beta);
 }
 
-// grid (ceil(N / 256), row tiles, batch); wavefront w of a workgroup takes 64 rows of W.
-template <int EPI>
+// grid (ceil(N / 256), row tiles, batch); wavefront w of a workgroup takes 64 rows of W and
+// RT tiles of 16 rows of x, which share every piece of W it loads (RT = 1 where a product has
+// few rows: decoding).
+template <int EPI, int RT>
 __global__ __launch_bounds__(256) void gemm_batched_kernel(BatchedParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g4 = lane >> 4;
@@ -65,12 +67,17 @@ __global__ __launch_bounds__(256) void gemm_batched_kernel(BatchedParams p) {
     first = p.offsets[b];
     count = p.offsets[b + 1] - first;
   }
-  const int m0 = blockIdx.y * 16;
+  const int m0 = blockIdx.y * 16 * RT;
   if (m0 >= count) return;
-  const int mine = min(m0 + r, count - 1);
-  const int dst_row = p.rows ? p.rows[first + mine] : mine;
-  const int src_row = p.rows ? dst_row / p.gather_div : mine;
-  const bf16_t* xr = p.x + (size_t)b * p.x_batch + (size_t)src_row * p.lda + g4 * 8;
+  int dst_row[RT];
+  const bf16_t* xr[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const int mine = min(m0 + t * 16 + r, count - 1);
+    dst_row[t] = p.rows ? p.rows[first + mine] : mine;
+    const int src_row = p.rows ? dst_row[t] / p.gather_div : mine;
+    xr[t] = p.x + (size_t)b * p.x_batch + (size_t)src_row * p.lda + g4 * 8;
+  }
   const bf16_t* wb = p.w + (size_t)b * p.w_batch;
   constexpr int SETS = EPI == BEPI_GATED ? 2 : 1;   // gate rows and up rows
   const bf16_t* wr[SETS][4];
@@ -79,49 +86,72 @@ __global__ __launch_bounds__(256) void gemm_batched_kernel(BatchedParams p) {
 #pragma unroll
     for (int t = 0; t < 4; ++t)
       wr[s][t] = wb + (size_t)(s * p.N + min(n0 + t * 16 + r, p.N - 1)) * p.K + g4 * 8;
-  f32x4 acc[SETS][4];
+  f32x4 acc[SETS][4][RT];
 #pragma unroll
   for (int s = 0; s < SETS; ++s)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[s][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int u = 0; u < RT; ++u) acc[s][t][u] = (f32x4){0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < p.K; k0 += 32) {
     const bool live = k0 + g4 * 8 < p.K;   // K is a multiple of 8: a lane's chunk is whole or absent
-    BFrag xf;
-    xf.u = live ? *(const uint4*)(xr + k0) : make_uint4(0, 0, 0, 0);
+    BFrag xf[RT];
+#pragma unroll
+    for (int u = 0; u < RT; ++u) xf[u].u = live ? *(const uint4*)(xr[u] + k0) : make_uint4(0, 0, 0, 0);
+    BFrag wf[SETS][4];
 #pragma unroll
     for (int s = 0; s < SETS; ++s)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        BFrag wf;
-        wf.u = live ? *(const uint4*)(wr[s][t] + k0) : make_uint4(0, 0, 0, 0);
-        acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf.v, acc[s][t], 0, 0, 0);
-      }
+      for (int t = 0; t < 4; ++t)
+        wf[s][t].u = live ? *(const uint4*)(wr[s][t] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < SETS; ++s)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int u = 0; u < RT; ++u)
+          acc[s][t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s][t].v, xf[u].v, acc[s][t][u], 0, 0, 0);
   }
-  if (m0 + r >= count) return;
-  // the lane holds outputs n0 + t * 16 + g4 * 4 + i of its row
-  if (EPI == BEPI_SCALED_F32) {
-    float* dst = (float*)p.out + (size_t)b * p.o_batch + (size_t)dst_row * p.ldo;
-    const float scale = p.row_scale ? p.row_scale[dst_row] : 1.f;
+  // the lane holds outputs n0 + t * 16 + g4 * 4 + i of its rows
+#pragma unroll
+  for (int u = 0; u < RT; ++u) {
+    if (m0 + u * 16 + r >= count) continue;
+    if (EPI == BEPI_SCALED_F32) {
+      float* dst = (float*)p.out + (size_t)b * p.o_batch + (size_t)dst_row[u] * p.ldo;
+      const float scale = p.row_scale ? p.row_scale[dst_row[u]] : 1.f;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int n = n0 + t * 16 + g4 * 4 + i;
+          if (n < p.N) dst[n] = acc[0][t][u][i] * scale;
+        }
+      continue;
+    }
+    bf16_t* dst = (bf16_t*)p.out + (size_t)b * p.o_batch + (size_t)dst_row[u] * p.ldo;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int n = n0 + t * 16 + g4 * 4 + i;
-        if (n < p.N) dst[n] = acc[0][t][i] * scale;
+        if (n >= p.N) continue;
+        const float v = EPI == BEPI_GATED ? batched_act(acc[0][t][u][i], acc[SETS - 1][t][u][i], p)
+                                          : acc[0][t][u][i];
+        dst[n] = f32_to_bf16(v);
       }
-    return;
   }
-  bf16_t* dst = (bf16_t*)p.out + (size_t)b * p.o_batch + (size_t)dst_row * p.ldo;
-#pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + t * 16 + g4 * 4 + i;
-      if (n >= p.N) continue;
-      const float v = EPI == BEPI_GATED ? batched_act(acc[0][t][i], acc[SETS - 1][t][i], p)
-                                        : acc[0][t][i];
-      dst[n] = f32_to_bf16(v);
-    }
+}
+
+// Row tiles per wavefront: four where a product has enough rows to fill them.
+template <int EPI>
+static void launch_batched(const BatchedParams& p, int max_rows, int batch, hipStream_t stream) {
+  if (max_rows > 32) {
+    dim3 grid((p.N + 255) / 256, (max_rows + 63) / 64, batch);
+    gemm_batched_kernel<EPI, 4><<<grid, 256, 0, stream>>>(p);
+  } else {
+    dim3 grid((p.N + 255) / 256, (max_rows + 15) / 16, batch);
+    gemm_batched_kernel<EPI, 1><<<grid, 256, 0, stream>>>(p);
+  }
 }
 
 static int batched_check(const BatchedParams& p, int batch, int max_tiles) {
@@ -148,8 +178,7 @@ extern "C" int mk_linear_batched_mfma(const void* x, const void* w, void* out, i
   if (batched_check(p, batch, tiles)) return 1;
   MK_REQUIRE(lda >= K && ldo >= N, "batched product: leading dimensions too small");
   if (M == 0) return 0;
-  dim3 grid((N + 255) / 256, tiles, batch);
-  gemm_batched_kernel<BEPI_BF16><<<grid, 256, 0, stream>>>(p);
+  launch_batched<BEPI_BF16>(p, M, batch, stream);
   MK_LAUNCH_CHECK("linear_batched_mfma");
   return 0;
 }
@@ -178,8 +207,7 @@ extern "C" int mk_expert_gated_mfma(const void* x, const void* w, void* act, con
   const int tiles = (max_rows + 15) / 16;
   if (batched_check(p, experts, tiles)) return 1;
   if (max_rows == 0) return 0;
-  dim3 grid((ff + 255) / 256, tiles, experts);
-  gemm_batched_kernel<BEPI_GATED><<<grid, 256, 0, stream>>>(p);
+  launch_batched<BEPI_GATED>(p, max_rows, experts, stream);
   MK_LAUNCH_CHECK("expert_gated_mfma");
   return 0;
 }
@@ -201,8 +229,7 @@ extern "C" int mk_expert_down_mfma(const void* act, const void* w, float* y, con
   const int tiles = (max_rows + 15) / 16;
   if (batched_check(p, experts, tiles)) return 1;
   if (max_rows == 0) return 0;
-  dim3 grid((N + 255) / 256, tiles, experts);
-  gemm_batched_kernel<BEPI_SCALED_F32><<<grid, 256, 0, stream>>>(p);
+  launch_batched<BEPI_SCALED_F32>(p, max_rows, experts, stream);
   MK_LAUNCH_CHECK("expert_down_mfma");
   return 0;
 }

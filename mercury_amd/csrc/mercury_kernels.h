@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 23
+#define MK_ABI_VERSION 24
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
@@ -275,6 +275,10 @@ int mk_expert_down_mfma(const void* act, const void* w, float* y, const int* row
 // mk_attention_mfma with one group of `heads`).  num_parts > 1 splits every tile's keys into
 // that many parts (at most mk_attention_latent_max_parts()) whose results part_o
 // [tiles, parts, dv, 16] / part_ml [tiles, parts, 2, 16] a second kernel merges.  No window.
+// Key and value widths come from a list of compiled shapes: mk_attention_latent_widths gives
+// the widths a cache must have for keys of at least dk and values of at least dv dims (host
+// pointers; returns 0 when no shape holds them), padded with zeros.
+int mk_attention_latent_widths(int dk, int dv, int* key_width, int* value_width);
 int mk_attention_latent_supported(int dk, int dv, int page_size);
 int mk_attention_latent_max_parts(void);
 int mk_attention_latent(const void* q, void* out, const void* k_cache, const void* v_cache,

@@ -240,6 +240,11 @@ void bind_ops(py::module_& m) {
     return blob(p);
   }, py::arg("w_gate_up"), py::arg("w_down"), py::arg("inter"), py::arg("act") = 0,
      py::arg("limit") = 0.f, py::arg("alpha") = 1.f, py::arg("beta") = 0.f);
+  m.def("latent_cache_widths", [](int key_dims, int value_dims) {
+    int key_width = 0, value_width = 0;
+    latent_cache_widths(key_dims, value_dims, key_width, value_width);
+    return py::make_tuple(key_width, value_width);
+  }, "Widths of the cache rows of an attention through a shared latent (keys, values).");
   m.def("latent_attention_params", [](const py::kwargs& kw) {
     const py::dict d = kw;
     LatentAttentionParams p;

@@ -241,4 +241,20 @@ std::string plan_defect(const AttentionPlan& plan, int head_dim, int page_size, 
   return t.mfma_error();
 }
 
+void latent_cache_widths(int key_dims, int value_dims, int& key_width, int& value_width) {
+  // (32-wide key chunks, 16-wide value tiles) of the shapes attention_latent.hip compiles, in
+  // its order; mk_attention_latent_supported has the last word at run time
+  static const int shapes[][2] = {{2, 2}, {2, 4}, {3, 4}, {4, 4}, {4, 8}, {5, 8}, {6, 8},
+                                  {8, 16}, {10, 16}, {12, 16}, {18, 32}, {20, 32}};
+  for (const auto& shape : shapes) {
+    if (key_dims <= shape[0] * 32 && value_dims <= shape[1] * 16) {
+      key_width = shape[0] * 32;
+      value_width = shape[1] * 16;
+      return;
+    }
+  }
+  key_width = (key_dims + 31) / 32 * 32;
+  value_width = (value_dims + 15) / 16 * 16;
+}
+
 }  // namespace mercury

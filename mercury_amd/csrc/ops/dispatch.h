@@ -58,6 +58,12 @@ bool folds_norm(int dtype, int m, int k);
 
 // ---- attention
 
+// The widths of the cache rows of an attention through a shared latent whose keys have
+// `key_dims` and whose values have `value_dims` dims: the first shape the matrix-core kernel
+// is compiled for that holds them (the rest of a row is zero), or, when none does, the dims
+// rounded up to multiples of 32 and 16 (the float32-arithmetic kernel then runs).
+void latent_cache_widths(int key_dims, int value_dims, int& key_width, int& value_width);
+
 struct AttentionPlan {
   bool mfma = false;
   int rows = 16;          // rows per wavefront tile

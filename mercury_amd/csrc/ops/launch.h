@@ -214,9 +214,17 @@ struct LatentArgs {
   void *k_cache = nullptr, *v_cache = nullptr;
   int page_size = 1;
   bool writes = true;
-  // rows as the cache holds them: padded to what the matrix-core attention takes
-  int key_width() const { return (kv_rank + rot + 31) / 32 * 32; }
-  int value_width() const { return (kv_rank + 15) / 16 * 16; }
+  // rows as the cache holds them: padded to a shape the matrix-core attention takes
+  int key_width() const {
+    int k, v;
+    latent_cache_widths(kv_rank + rot, kv_rank, k, v);
+    return k;
+  }
+  int value_width() const {
+    int k, v;
+    latent_cache_widths(kv_rank + rot, kv_rank, k, v);
+    return v;
+  }
 };
 // Down-projection, norms, rotation and cache write, query up-projection; the queries come back
 // as rows [heads, kv_rank + rot] = [absorbed | rotated].

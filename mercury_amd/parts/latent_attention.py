@@ -57,10 +57,8 @@ class LatentAttention(Mixer):
         self._alone: dict = {}
 
     def cache_spec(self) -> CacheSpec:
-        # one shared head; rows padded to what the matrix-core attention takes (key rows to a
-        # multiple of 32, the transposed values to a multiple of 16), the padding zero
-        key_width = -(-(self.kv_rank + self.rot_dim) // 32) * 32
-        value_width = -(-self.kv_rank // 16) * 16
+        # one shared head; rows padded with zeros to a shape the matrix-core attention takes
+        key_width, value_width = core.latent_cache_widths(self.kv_rank + self.rot_dim, self.kv_rank)
         return CacheSpec(1, key_width, self.window, value_dim=value_width)
 
     def param_specs(self) -> dict:
