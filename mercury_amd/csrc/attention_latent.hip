@@ -63,8 +63,17 @@ struct LatentAttnParams {
 // The wavefronts of a workgroup are independent (tile, part) units; the block size is a
 // launch parameter (one wavefront a workgroup when there are few units, so that they spread
 // over the compute units).
+// Whether a shape's registers hold a block's keys and values at once beside the queries and
+// the accumulators.  The shapes that do not keep their queries in LDS (each wavefront its own
+// 16 rows, written and read by the same lanes: no barrier), take a block's keys half by half
+// and its values after them, and so fit two wavefronts a SIMD.
+constexpr bool latent_early(int dkc, int dvt) { return dkc * 12 + dvt * 8 <= 320; }
+constexpr int latent_q_stride(int dkc) { return dkc * 32 + 8; }   // elements; 16 bytes of padding
+
+extern __shared__ __align__(16) unsigned char latent_lds[];
+
 template <int DKC, int DVT>
-__global__ __launch_bounds__(256) void attn_latent_kernel(LatentAttnParams p) {
+__global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 1 : 2)) void attn_latent_kernel(LatentAttnParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int unit = blockIdx.x * (blockDim.x >> 6) + wave;
   if (unit >= p.num_tiles * p.num_parts) return;   // a whole wavefront; nothing is shared
@@ -90,11 +99,16 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(LatentAttnParams p) {
   constexpr int DK = DKC * 32, DV = DVT * 16;
   const int* table = p.block_table + (size_t)seq * p.table_stride;
 
-  LFrag qf[DKC];
+  constexpr bool EARLY = latent_early(DKC, DVT);
+  LFrag qf[EARLY ? DKC : 1];
+  bf16_t* qs = (bf16_t*)latent_lds + ((size_t)wave * 16 + r) * latent_q_stride(DKC) + g4 * 8;
   {
     const bf16_t* qrow = p.q + ((size_t)token * p.heads + head) * DK + g4 * 8;
 #pragma unroll
-    for (int c = 0; c < DKC; ++c) qf[c].u = *(const uint4*)(qrow + c * 32);
+    for (int c = 0; c < DKC; ++c) {
+      if constexpr (EARLY) qf[c].u = *(const uint4*)(qrow + c * 32);
+      else *(uint4*)(qs + c * 32) = *(const uint4*)(qrow + c * 32);
+    }
   }
   f32x4 acc[DVT];
 #pragma unroll
@@ -118,7 +132,6 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(LatentAttnParams p) {
     }
     // Everything the block needs is asked for before the first product where the registers
     // hold it all; the widest shapes take the keys half by half and the values after them.
-    constexpr bool EARLY = DKC * 12 + DVT * 8 <= 320;
     LFrag vf[DVT];
     float s[8];
     if constexpr (EARLY) {
@@ -149,14 +162,18 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(LatentAttnParams p) {
         for (int c = 0; c < DKC; ++c) kf[c].u = *(const uint4*)(kbase[h] + c * 32);
         f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < DKC; ++c)
-          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c].v, qf[c].v, sc, 0, 0, 0);
+        for (int c = 0; c < DKC; ++c) {
+          LFrag qc;
+          qc.u = *(const uint4*)(qs + c * 32);
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c].v, qc.v, sc, 0, 0, 0);
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) s[h * 4 + i] = sc[i];
         __builtin_amdgcn_sched_barrier(0);   // the next loads stay behind these products
       }
+      // (the values: half of them now, the other half behind the first half's products)
 #pragma unroll
-      for (int t = 0; t < DVT; ++t) {
+      for (int t = 0; t < DVT / 2; ++t) {
         vf[t].u2[0] = *(const uint2*)(vbase[0] + (size_t)t * 16 * ps);
         vf[t].u2[1] = *(const uint2*)(vbase[1] + (size_t)t * 16 * ps);
       }
@@ -188,9 +205,26 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(LatentAttnParams p) {
     LFrag pf;
     pf.u = make_uint4(pack_bf16x2(e[0], e[1]), pack_bf16x2(e[2], e[3]), pack_bf16x2(e[4], e[5]),
                       pack_bf16x2(e[6], e[7]));
+    if constexpr (EARLY) {
 #pragma unroll
-    for (int t = 0; t < DVT; ++t)
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pf.v, acc[t], 0, 0, 0);
+      for (int t = 0; t < DVT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pf.v, acc[t], 0, 0, 0);
+    } else {
+      static_assert(EARLY || DVT % 2 == 0, "the values of a wide shape go in two halves");
+#pragma unroll
+      for (int t = 0; t < DVT / 2; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pf.v, acc[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < DVT / 2; ++t) {
+        vf[t].u2[0] = *(const uint2*)(vbase[0] + (size_t)(t + DVT / 2) * 16 * ps);
+        vf[t].u2[1] = *(const uint2*)(vbase[1] + (size_t)(t + DVT / 2) * 16 * ps);
+      }
+#pragma unroll
+      for (int t = 0; t < DVT / 2; ++t)
+        acc[t + DVT / 2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pf.v, acc[t + DVT / 2], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
   // a row's sum lies in its four lanes
   lsum += __shfl_xor(lsum, 16, 64);
@@ -219,6 +253,130 @@ __global__ __launch_bounds__(256) void attn_latent_kernel(LatentAttnParams p) {
   }
 }
 
+// The widest shapes with the keys split into parts (decoding: few tiles, long ranges of keys):
+// the four wavefronts of a workgroup take one (tile, part) together.  Each computes all the
+// scores (the keys' second to fourth reading comes from the caches) but only its quarter of
+// the value tiles, so its registers hold a block's keys and its values at once and every load
+// of a block is on its way before the first product: one trip to memory a block, where the
+// kernel above, alone with all value tiles, makes four.
+template <int DKC, int DVT>
+__global__ __launch_bounds__(256) void attn_latent_split_values_kernel(LatentAttnParams p) {
+  static_assert(DVT % 4 == 0, "four wavefronts share the value tiles");
+  constexpr int MINE = DVT / 4;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = blockIdx.x;
+  const int tile = p.num_tiles - 1 - unit / p.num_parts;
+  const int part = unit % p.num_parts;
+  const int r = lane & 15, g4 = lane >> 4;
+  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
+  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  const int kv_len = p.kv_len[seq];
+  const int rows = q_len * p.heads;
+  const int f = min(row0 + r, rows - 1);
+  const int token = q0 + f / p.heads, head = f % p.heads;
+  const int pos = kv_len - q_len + f / p.heads;
+  const int last_row = min(row0 + 15, rows - 1);
+  const int kmax = kv_len - q_len + last_row / p.heads;
+  const int all_see = kv_len - q_len + row0 / p.heads;
+  const int blocks = (kmax >> 5) + 1;
+  const int per = (blocks + p.num_parts - 1) / p.num_parts;
+  const int b_begin = part * per, b_end = min(blocks, b_begin + per);
+  const int ps = 1 << p.page_shift;
+  constexpr int DK = DKC * 32, DV = DVT * 16;
+  const int* table = p.block_table + (size_t)seq * p.table_stride;
+
+  LFrag qf[DKC];
+  {
+    const bf16_t* qrow = p.q + ((size_t)token * p.heads + head) * DK + g4 * 8;
+#pragma unroll
+    for (int c = 0; c < DKC; ++c) qf[c].u = *(const uint4*)(qrow + c * 32);
+  }
+  f32x4 acc[MINE];
+#pragma unroll
+  for (int t = 0; t < MINE; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+  const float c2 = p.scale_log2;
+
+  for (int b = b_begin; b < b_end; ++b) {
+    const int key0 = b << 5;
+    const bf16_t* kbase[2];
+    const bf16_t* vbase[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int kh = key0 + h * 16;
+      const int index = kh >> p.page_shift;
+      const int page = index < p.table_stride ? max(table[index], 0) : 0;
+      const int off = kh & (ps - 1);
+      kbase[h] = p.k_cache + ((size_t)page * ps + off + r) * DK + g4 * 8;
+      vbase[h] = p.v_cache + ((size_t)page * DV + wave * MINE * 16 + r) * ps + off + g4 * 4;
+    }
+    LFrag kf[2][DKC];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int c = 0; c < DKC; ++c) kf[h][c].u = *(const uint4*)(kbase[h] + c * 32);
+    LFrag vf[MINE];
+#pragma unroll
+    for (int t = 0; t < MINE; ++t) {
+      vf[t].u2[0] = *(const uint2*)(vbase[0] + (size_t)t * 16 * ps);
+      vf[t].u2[1] = *(const uint2*)(vbase[1] + (size_t)t * 16 * ps);
+    }
+    float s[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DKC; ++c)
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[h][c].v, qf[c].v, sc, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[h * 4 + i] = sc[i];
+    }
+    if (key0 + 31 > all_see) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (key0 + h * 16 + g4 * 4 + i > pos) s[h * 4 + i] = -INFINITY;
+    }
+    float bm = c2 * fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                          fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+      bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+      const float m_new = fmaxf(m, bm);
+      const float corr = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
+      lsum *= corr;
+#pragma unroll
+      for (int t = 0; t < MINE; ++t) acc[t] *= corr;
+      m = m_new;
+    }
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], c2, -m_use));
+    lsum += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+    LFrag pf;
+    pf.u = make_uint4(pack_bf16x2(e[0], e[1]), pack_bf16x2(e[2], e[3]), pack_bf16x2(e[4], e[5]),
+                      pack_bf16x2(e[6], e[7]));
+#pragma unroll
+    for (int t = 0; t < MINE; ++t)
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pf.v, acc[t], 0, 0, 0);
+  }
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+  float* po = p.part_o + ((size_t)tile * p.num_parts + part) * DV * 16;
+#pragma unroll
+  for (int t = 0; t < MINE; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      po[(size_t)((wave * MINE + t) * 16 + g4 * 4 + i) * 16 + r] = acc[t][i];
+  if (wave == 0 && g4 == 0) {   // every wavefront has the same maxima and sums
+    float* ml = p.part_ml + ((size_t)tile * p.num_parts + part) * 32;
+    ml[r] = m;
+    ml[16 + r] = lsum;
+  }
+}
+
 #define LATENT_MAX_PARTS 64
 
 // grid (tiles, value tiles / 4): a workgroup adds up the parts' results of 64 dims of a tile's
@@ -232,30 +390,59 @@ __global__ __launch_bounds__(256) void attn_latent_merge_kernel(LatentAttnParams
   const int rows = q_len * p.heads;
   const int dv = p.dvt * 16;
   const float* ml = p.part_ml + (size_t)tile * p.num_parts * 32;
+  // the parts' weights: thread (part, row) first, then one thread a row for the maximum
+  for (int i = threadIdx.x; i < p.num_parts * 16; i += blockDim.x)
+    weight[i >> 4][i & 15] = ml[(i >> 4) * 32 + (i & 15)];
+  __syncthreads();
   if (threadIdx.x < 16) {
     const int r = threadIdx.x;
     float m = -INFINITY;
-    for (int s = 0; s < p.num_parts; ++s) m = fmaxf(m, ml[s * 32 + r]);
+    for (int s = 0; s < p.num_parts; ++s) m = fmaxf(m, weight[s][r]);
+    inv[r] = m;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < p.num_parts * 16; i += blockDim.x) {
+    const float ms = weight[i >> 4][i & 15];
+    weight[i >> 4][i & 15] = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - inv[i & 15]);
+  }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    const int r = threadIdx.x;
     float total = 0.f;
-    for (int s = 0; s < p.num_parts; ++s) {
-      const float ms = ml[s * 32 + r];
-      const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m);
-      weight[s][r] = w;
-      total += w * ml[s * 32 + 16 + r];
-    }
+    for (int s = 0; s < p.num_parts; ++s) total += weight[s][r] * ml[s * 32 + 16 + r];
     inv[r] = 1.f / total;
   }
   __syncthreads();
+  // 64 dims x 16 rows = 1024 values a workgroup, four a thread, the parts' loads eight deep
   const float* po = p.part_o + (size_t)tile * p.num_parts * dv * 16;
-  // 64 dims x 16 rows = 1024 values, four a thread
-  for (int idx = blockIdx.y * 1024 + threadIdx.x; idx < min(dv * 16, (int)(blockIdx.y + 1) * 1024);
-       idx += 256) {
+  const size_t stride = (size_t)dv * 16;
+  const int base = blockIdx.y * 1024 + threadIdx.x;
+  float total[4] = {0.f, 0.f, 0.f, 0.f};
+  int s = 0;
+  for (; s + 8 <= p.num_parts; s += 8) {
+    float v[8][4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        v[j][k] = base + k * 256 < dv * 16 ? po[(size_t)(s + j) * stride + base + k * 256] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) total[k] += weight[s + j][(base + k * 256) & 15] * v[j][k];
+  }
+  for (; s < p.num_parts; ++s)
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (base + k * 256 < dv * 16)
+        total[k] += weight[s][(base + k * 256) & 15] * po[(size_t)s * stride + base + k * 256];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int idx = base + k * 256;
     const int d = idx >> 4, r = idx & 15;
-    if (row0 + r >= rows) continue;
-    float total = 0.f;
-    for (int s = 0; s < p.num_parts; ++s) total += weight[s][r] * po[(size_t)s * dv * 16 + idx];
+    if (idx >= dv * 16 || row0 + r >= rows) continue;
     const int f = row0 + r;
-    p.out[((size_t)(q0 + f / p.heads) * p.heads + f % p.heads) * dv + d] = f32_to_bf16(total * inv[r]);
+    p.out[((size_t)(q0 + f / p.heads) * p.heads + f % p.heads) * dv + d] = f32_to_bf16(total[k] * inv[r]);
   }
 }
 
@@ -323,9 +510,19 @@ extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache
   const int waves = units >= 2048 ? LAT_WAVES : 1;
   MK_REQUIRE((units + waves - 1) / waves < (1ll << 31), "latent attention: too many tiles");
   const dim3 grid((unsigned)((units + waves - 1) / waves));
-#define LATENT_LAUNCH(C, T)                                                   \
-  if (dk == (C) * 32 && dv == (T) * 16)                                       \
-    attn_latent_kernel<C, T><<<grid, 64 * waves, 0, stream>>>(p);
+  if (num_parts > 1 && dv == 512 && (dk == 576 || dk == 640)) {
+    if (dk == 576) attn_latent_split_values_kernel<18, 32><<<(unsigned)units, 256, 0, stream>>>(p);
+    else attn_latent_split_values_kernel<20, 32><<<(unsigned)units, 256, 0, stream>>>(p);
+    MK_LAUNCH_CHECK("attention_latent");
+    attn_latent_merge_kernel<<<dim3(num_tiles, (p.dvt + 3) / 4), 256, 0, stream>>>(p);
+    MK_LAUNCH_CHECK("attention_latent_merge");
+    return 0;
+  }
+#define LATENT_LAUNCH(C, T)                                                                  \
+  if (dk == (C) * 32 && dv == (T) * 16)                                                      \
+    attn_latent_kernel<C, T><<<grid, 64 * waves,                                             \
+                               latent_early(C, T) ? 0 : waves * 16 * latent_q_stride(C) * 2, \
+                               stream>>>(p);
   LATENT_SHAPES(LATENT_LAUNCH)
 #undef LATENT_LAUNCH
   MK_LAUNCH_CHECK("attention_latent");

@@ -198,21 +198,26 @@ int run_parallel(const void* params, mk_op_context* ctx) {
   const ParallelParams& p = *static_cast<const ParallelParams*>(params);
   const long long n = (long long)ctx->step->num_tokens * ctx->hidden;
   float* const h = ctx->h;
+  // A factor of one needs no buffer: the sublayers add into the stream itself, and what they
+  // leave as partial sums is passed on (the first) or added here (any further ones).
+  const bool direct = p.mult == 1.f;
   float* y = nullptr;
-  int code = guarded(ctx, [&] {
-    Launch l(ctx);
-    y = zeros(l, n);
-  });
-  if (code) return code;
+  if (!direct) {
+    const int code = guarded(ctx, [&] {
+      Launch l(ctx);
+      y = zeros(l, n);
+    });
+    if (code) return code;
+  }
   const float* parts[kParallelMax] = {nullptr};
   int counts[kParallelMax] = {0};
   for (int i = 0; i < p.count; ++i) {
-    ctx->h = y;
+    ctx->h = direct ? h : y;
     ctx->out_x = nullptr;
     ctx->out_x_rows = ctx->out_x_live = 0;
     ctx->out_pending = nullptr;
     ctx->out_pending_count = 0;
-    code = p.sub[i].run(static_cast<const char*>(params) + p.sub[i].offset, ctx);
+    const int code = p.sub[i].run(static_cast<const char*>(params) + p.sub[i].offset, ctx);
     ctx->h = h;
     if (code) return code;
     parts[i] = ctx->out_pending;
@@ -225,15 +230,22 @@ int run_parallel(const void* params, mk_op_context* ctx) {
   ctx->out_logits_ready = 0;
   return guarded(ctx, [&] {
     Launch l(ctx);
-    // partial sums of at most two sublayers go into the sum directly; any further ones first
-    // into y
     int first = -1, second = -1;
     for (int i = 0; i < p.count; ++i) {
       if (!counts[i]) continue;
       if (first < 0) first = i;
       else if (second < 0) second = i;
-      else scaled_add(l, y, nullptr, parts[i], counts[i], nullptr, 0, n, 1.f);
+      else scaled_add(l, direct ? h : y, nullptr, parts[i], counts[i], nullptr, 0, n, 1.f);
     }
+    if (direct) {
+      if (second >= 0) scaled_add(l, h, nullptr, parts[second], counts[second], nullptr, 0, n, 1.f);
+      if (first >= 0) {
+        ctx->out_pending = parts[first];
+        ctx->out_pending_count = counts[first];
+      }
+      return;
+    }
+    // partial sums of at most two sublayers go into the sum directly
     scaled_add(l, h, y, first < 0 ? nullptr : parts[first], first < 0 ? 0 : counts[first],
                second < 0 ? nullptr : parts[second], second < 0 ? 0 : counts[second], n, p.mult);
   });

@@ -461,7 +461,7 @@ Queries latent_queries(Launch& l, const void* x, int m, int hidden, const Latent
 namespace {
 // Decoding with few tiles: the keys are cut into parts until about this many wavefronts run,
 // a part being at least this many blocks of 32 keys.
-constexpr int kLatentWaves = 512;
+constexpr int kLatentWaves = 1024;
 constexpr int kLatentMinBlocks = 4;
 }  // namespace
 
