@@ -4,10 +4,11 @@
 // its own per head needs (x[t, head, :] W[head]^T), and, with a list of rows per product, what
 // routed experts need (every expert's matrix over the tokens routed to it).
 //
-// A wavefront computes 16 rows of x against 64 rows of W: W is the A operand (a lane holds 8
-// consecutive k of one row of W), x^T the B operand, so a lane ends up with four consecutive
-// outputs of one row of x.  Operands go from memory straight into the products; the matrices
-// are small enough (a head's, an expert's) to stay in the caches across the row tiles.
+// A wavefront computes one or four tiles of 16 rows of x against 64 rows of W: W is the A
+// operand (a lane holds 8 consecutive k of one row of W), x^T the B operand, so a lane ends up
+// with four consecutive outputs of a row of x, and the row tiles share every piece of W the
+// wavefront loads.  Operands go from memory straight into the products; the matrices are
+// small enough (a head's, an expert's) to stay in the caches across the workgroups.
 // K must be a multiple of 8 (a lane's 16 bytes); a last chunk of K short of 32 is padded with
 // zeros in registers.
 //

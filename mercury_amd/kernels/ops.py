@@ -617,3 +617,32 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tenso
                                   _ptr(top_ps), _ptr(uniforms), _ptr(scratch), _ptr(out),
                                   _stream()), "sample")
     return out
+
+
+def scaled_add(h: torch.Tensor, y: torch.Tensor | None, mult: float, a: torch.Tensor | None = None,
+               b: torch.Tensor | None = None) -> torch.Tensor:
+    """h += mult * (y + a.sum(0) + b.sum(0)) in place: h and y float32 [T, H], a and b float32
+    partial sums [P, T, H] (any of y, a, b may be None)."""
+    _dev(h, y, a, b)
+    for t in (h, y, a, b):
+        if t is not None and t.dtype != torch.float32:
+            raise KernelArgumentError("scaled_add works on float32 tensors")
+    n = h.numel()
+    for t, lead in ((y, 0), (a, 1), (b, 1)):
+        if t is not None and t.numel() != n * (t.shape[0] if lead else 1):
+            raise KernelArgumentError("scaled_add: shapes do not match the stream's")
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_scaled_add(h.data_ptr(), _ptr(y), _ptr(a), 0 if a is None else a.shape[0],
+                                      _ptr(b), 0 if b is None else b.shape[0], n, float(mult), n,
+                                      _stream()), "scaled_add")
+    return h
+
+
+def zeros_like_stream(h: torch.Tensor) -> torch.Tensor:
+    """A zeroed float32 buffer of the stream's shape, filled by a kernel (safe under a graph
+    capture, which records no memset)."""
+    _dev(h)
+    out = torch.empty_like(h, dtype=torch.float32)
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_fill_zero(out.data_ptr(), out.numel(), _stream()), "fill_zero")
+    return out

@@ -15,8 +15,8 @@ from __future__ import annotations
 
 from ..config.model_config import TalolornConfig
 from ..config.registry import register_architecture
-from ..parts import (DecoderModel, GatedMLP, LatentAttention, LayerCall, ParallelBlock, RMSNorm,
-                     RotaryPosition, RoutedExperts, TokenEmbedding)
+from ..parts import (DecoderModel, GatedMLP, LatentAttention, LayerCall, NoPosition, ParallelBlock,
+                     RMSNorm, RotaryPosition, RoutedExperts, TokenEmbedding)
 
 PART_NAMES = {"mixer": "mix.", "ffn": "mlp.", "norm": "norm1."}
 FF_NAMES = {"gate": "gate", "up": "up", "down": "down"}
@@ -42,19 +42,16 @@ def _feed_forward(cfg: TalolornConfig, ff):
 @register_architecture("Talolorn", TalolornConfig)
 def build_talolorn(cfg: TalolornConfig) -> DecoderModel:
     layers, layer_ids, place = [], [], {}
-    rotaries: dict = {}    # one angle table per (width, base, turned dims)
+    positions: dict = {}    # one angle table per (width, base, turned dims)
     for i, entry in enumerate(cfg.layers):
         if entry.weights_of is not None:
             continue
         m = entry.mixer
         key = (m.rot_dim, m.rot_base, m.rot_dims)
-        if key not in rotaries:
-            rotaries[key] = RotaryPosition(max(m.rot_dim, 2), m.rot_base, rotary_dim=m.rot_dims or 2,
-                                           interleaved=True) if m.rot_dims else None
-        position = rotaries[key]
-        if position is None:
-            from ..parts import NoPosition
-            position = NoPosition()
+        if key not in positions:
+            positions[key] = (RotaryPosition(m.rot_dim, m.rot_base, rotary_dim=m.rot_dims,
+                                             interleaved=True) if m.rot_dims else NoPosition())
+        position = positions[key]
         mixer = LatentAttention(cfg.width, m.heads, m.dim, m.rot_dim, m.vdim, m.q_rank, m.kv_rank,
                                 position, eps=cfg.norm_eps, scale=m.scale)
         place[i] = len(layers)

@@ -2,9 +2,8 @@
 
 from __future__ import annotations
 
-import torch
-
 from ..hostcore import core
+from ..kernels import ops
 from .base import FeedForward, Mixer, Norm, Part
 from .lowering import OneOp
 
@@ -172,10 +171,8 @@ class ParallelBlock(Part):
             return left
         # a sublayer that stays with Python: the same sum, put together here
         x = self.norm.forward(h, dtype, partials=pending)
-        y = torch.zeros_like(h)
-        for left in (self.mixer.forward(x, step, cache, state, y),
-                     None if self.ffn is None else self.ffn.forward(x, step, y)):
-            if left is not None:
-                y += left.sum(dim=0)
-        h.add_(y, alpha=self.residual_mult)
+        y = ops.zeros_like_stream(h)
+        left_mixer = self.mixer.forward(x, step, cache, state, y)
+        left_ffn = None if self.ffn is None else self.ffn.forward(x, step, y)
+        ops.scaled_add(h, y, self.residual_mult, left_mixer, left_ffn)
         return None

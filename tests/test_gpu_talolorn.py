@@ -170,6 +170,51 @@ def test_clamped_gate_feed_forward_alone(dtype, rows):
         GatedMLP(8, 8, activation="swish_clamp")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mult", [1.0, 0.6])
+def test_parallel_block_around_the_other_mixer_and_feed_forward(dtype, mult):
+    """The arrangement alone, with the package's ordinary attention and SiLU-gated projection as
+    its sublayers: x + m * (mixer(norm(x)) + ff(norm(x))), over two portions."""
+    from mercury_amd.cache import CacheManager
+    from mercury_amd.engine.batch import SeqChunk, build_step
+    from mercury_amd.parts import (Attention, GatedMLP, LayerCache, ParallelBlock, RMSNorm,
+                                   RotaryPosition)
+    from tests.plain import qwen2_plain
+
+    hidden, n_q, n_kv, d, page = 64, 4, 2, 16, 16
+    block = ParallelBlock(Attention(hidden, n_q, n_kv, d, RotaryPosition(d, 10000.0), qkv_bias=True),
+                          GatedMLP(hidden, 96), RMSNorm(hidden, 1e-6),
+                          {"mixer": "attn.", "ffn": "mlp.", "norm": "norm."}, residual_mult=mult)
+    params = bind_random(block, dtype, scale=0.1, seed=50)
+    block.prepare(64, DEV)
+    manager = CacheManager({0: block.mixer.cache_spec()}, 8, page, 2)
+    cache = LayerCache(torch.zeros(8, n_kv, page, d, dtype=dtype, device=DEV),
+                       torch.zeros(8, n_kv, d, page, dtype=dtype, device=DEV), 0, page, True)
+    x = rnd(30, hidden, seed=31)
+    out = []
+    for start, count in ((0, 19), (19, 11)):
+        if not manager.holds("s"):
+            manager.admit("s", [], count)
+        manager.grow("s", start, start + count)
+        step = build_step([SeqChunk("s", [0] * count, start, [])], manager, 10, 4096, DEV)
+        h = x[start:start + count].to(DEV).contiguous()
+        settle(h, block.forward(h, step, cache, None, dtype))
+        out.append(h.cpu())
+
+    def plain_block(cast_dtype):
+        w = {k: v.to(cast_dtype) for k, v in params.items()}
+        normed, _ = qwen2_plain.rms_norm(x.to(cast_dtype), w["norm.weight"], 1e-6)
+        cos, sin = qwen2_plain.rotary_table(d, range(30), 10000.0)
+        cfg = {"num_attention_heads": n_q, "num_key_value_heads": n_kv, "head_dim": d}
+        attn = {k[len("attn."):]: v for k, v in w.items() if k.startswith("attn.")}
+        mixed = qwen2_plain.attention_layer(normed, attn, "", cfg, cos, sin, None)
+        ff = qwen2_plain.gated_mlp(normed, w["mlp.gate_proj.weight"], w["mlp.up_proj.weight"],
+                                   w["mlp.down_proj.weight"])
+        return x + mult * (mixed.float() + ff.float())
+
+    close(torch.cat(out), plain_block(torch.float32), dtype, plain_block(torch.bfloat16))
+
+
 # ---------------------------------------------------------------------------- whole models
 
 
