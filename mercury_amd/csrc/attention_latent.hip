@@ -377,6 +377,180 @@ __global__ __launch_bounds__(256) void attn_latent_split_values_kernel(LatentAtt
   }
 }
 
+// Prompt portions: a workgroup takes a tile of 64 rows of one sequence, 16 a wavefront, and
+// walks the keys once for all four: every block of 32 keys and its transposed values are
+// brought into LDS by the whole workgroup (through registers) and read from there by each
+// wavefront as its operands, so a block costs the L2 one reading for 64 rows instead of four.
+// One buffer; two workgroups a compute unit, one multiplying while the other loads.  Key rows
+// lie 16 bytes, value rows 16 bytes further apart than their width, against bank conflicts.
+template <int DKC, int DVT>
+__global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 2 : 1)) void attn_latent_staged_kernel(LatentAttnParams p) {
+  constexpr int DK = DKC * 32, DV = DVT * 16;
+  constexpr int KS = DK + 8, VS = 40;                 // row pitches in elements
+  __shared__ __align__(16) bf16_t ks[32 * KS];
+  __shared__ __align__(16) bf16_t vs[DV * VS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g4 = lane >> 4;
+  const int tile = p.num_tiles - 1 - blockIdx.x;     // the longest walks start first
+  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
+  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  const int kv_len = p.kv_len[seq];
+  const int rows = q_len * p.heads;
+  const int first_pos = kv_len - q_len;
+  const int my_row0 = row0 + wave * 16;
+  const bool wave_live = my_row0 < rows;             // a tile's last wavefronts may have no rows
+  const int f = min(my_row0 + r, rows - 1);
+  const bool row_ok = my_row0 + r < rows;
+  const int token = q0 + f / p.heads, head = f % p.heads;
+  const int pos = first_pos + f / p.heads;
+  const int my_kmax = first_pos + min(my_row0 + 15, rows - 1) / p.heads;
+  const int all_see = first_pos + min(my_row0, rows - 1) / p.heads;
+  const int blocks = ((first_pos + min(row0 + 63, rows - 1) / p.heads) >> 5) + 1;
+  const int ps = 1 << p.page_shift;
+  const int* table = p.block_table + (size_t)seq * p.table_stride;
+
+  LFrag qf[DKC];
+  {
+    const bf16_t* qrow = p.q + ((size_t)token * p.heads + head) * DK + g4 * 8;
+#pragma unroll
+    for (int c = 0; c < DKC; ++c) qf[c].u = *(const uint4*)(qrow + c * 32);
+  }
+  f32x4 acc[DVT];
+#pragma unroll
+  for (int t = 0; t < DVT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+  const float c2 = p.scale_log2;
+  constexpr int K_CHUNKS = 32 * (DK / 8), V_CHUNKS = DV * 4;   // 16-byte pieces of a block
+  constexpr int K_MINE = (K_CHUNKS + 255) / 256, V_MINE = (V_CHUNKS + 255) / 256;
+
+  for (int b = 0; b < blocks; ++b) {
+    const int key0 = b << 5;
+    // the two halves' places in the cache (scalars: an array indexed by the half would live
+    // in scratch memory)
+    const int index0 = key0 >> p.page_shift, index1 = (key0 + 16) >> p.page_shift;
+    const int page0 = index0 < p.table_stride ? max(table[index0], 0) : 0;
+    const int page1 = index1 < p.table_stride ? max(table[index1], 0) : 0;
+    const int off0 = key0 & (ps - 1), off1 = (key0 + 16) & (ps - 1);
+    // (a thread past the last piece repeats it: loads and stores without conditions)
+#define LAT_K_FROM(i, dst)                                                                        \
+  {                                                                                               \
+    const int idx_ = min(tid + (i) * 256, K_CHUNKS - 1);                                          \
+    const int key_ = idx_ / (DK / 8), ch_ = idx_ % (DK / 8);                                      \
+    const size_t slot_ = key_ < 16 ? (size_t)page0 * ps + off0 + key_                             \
+                                   : (size_t)page1 * ps + off1 + key_ - 16;                       \
+    dst = *(const uint4*)(p.k_cache + slot_ * DK + ch_ * 8);                                      \
+  }
+#define LAT_K_TO(i, src)                                                                          \
+  {                                                                                               \
+    const int idx_ = min(tid + (i) * 256, K_CHUNKS - 1);                                          \
+    *(uint4*)(ks + (idx_ / (DK / 8)) * KS + (idx_ % (DK / 8)) * 8) = src;                         \
+  }
+#define LAT_V_FROM(i, dst)                                                                        \
+  {                                                                                               \
+    const int idx_ = min(tid + (i) * 256, V_CHUNKS - 1);                                          \
+    const bool second_ = (idx_ >> 1) & 1;                                                         \
+    dst = *(const uint4*)(p.v_cache + ((size_t)(second_ ? page1 : page0) * DV + (idx_ >> 2)) * ps + \
+                          (second_ ? off1 : off0) + (idx_ & 1) * 8);                              \
+  }
+#define LAT_V_TO(i, src)                                                                          \
+  {                                                                                               \
+    const int idx_ = min(tid + (i) * 256, V_CHUNKS - 1);                                          \
+    *(uint4*)(vs + (idx_ >> 2) * VS + ((idx_ >> 1) & 1) * 16 + (idx_ & 1) * 8) = src;             \
+  }
+    // (named registers, not arrays: the compiler keeps such arrays in scratch memory here)
+    static_assert(K_MINE <= 10 && V_MINE <= 8, "more pieces a thread than it has names for");
+    uint4 k0, k1, k2, k3, k4, k5, k6, k7, k8, k9, v0, v1, v2, v3, v4, v5, v6, v7;
+#define LAT_EACH_K(DO) DO(0, k0) DO(1, k1) DO(2, k2) DO(3, k3) DO(4, k4) DO(5, k5) DO(6, k6) DO(7, k7) DO(8, k8) DO(9, k9)
+#define LAT_EACH_V(DO) DO(0, v0) DO(1, v1) DO(2, v2) DO(3, v3) DO(4, v4) DO(5, v5) DO(6, v6) DO(7, v7)
+#define LAT_KF(i, reg) if constexpr (i < K_MINE) LAT_K_FROM(i, reg)
+#define LAT_KT(i, reg) if constexpr (i < K_MINE) LAT_K_TO(i, reg)
+#define LAT_VF(i, reg) if constexpr (i < V_MINE) LAT_V_FROM(i, reg)
+#define LAT_VT(i, reg) if constexpr (i < V_MINE) LAT_V_TO(i, reg)
+    if constexpr (latent_early(DKC, DVT)) {
+      LAT_EACH_K(LAT_KF)
+      LAT_EACH_V(LAT_VF)
+      __syncthreads();     // whoever still reads the block before has finished
+      LAT_EACH_K(LAT_KT)
+      LAT_EACH_V(LAT_VT)
+    } else {               // the widest shapes: keys, then values, for the registers' sake
+      LAT_EACH_K(LAT_KF)
+      __syncthreads();
+      LAT_EACH_K(LAT_KT)
+      __builtin_amdgcn_sched_barrier(0);
+      LAT_EACH_V(LAT_VF)
+      LAT_EACH_V(LAT_VT)
+    }
+#undef LAT_EACH_K
+#undef LAT_EACH_V
+#undef LAT_KF
+#undef LAT_KT
+#undef LAT_VF
+#undef LAT_VT
+#undef LAT_K_FROM
+#undef LAT_K_TO
+#undef LAT_V_FROM
+#undef LAT_V_TO
+    __syncthreads();
+    if (!wave_live || key0 > my_kmax) continue;      // the wavefront's rows see nothing here
+    float s[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DKC; ++c) {
+        LFrag kf;
+        kf.u = *(const uint4*)(ks + (h * 16 + r) * KS + c * 32 + g4 * 8);
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[h * 4 + i] = sc[i];
+    }
+    if (key0 + 31 > all_see) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (key0 + h * 16 + g4 * 4 + i > pos) s[h * 4 + i] = -INFINITY;
+    }
+    float bm = c2 * fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                          fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+      bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+      const float m_new = fmaxf(m, bm);
+      const float corr = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
+      lsum *= corr;
+#pragma unroll
+      for (int t = 0; t < DVT; ++t) acc[t] *= corr;
+      m = m_new;
+    }
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], c2, -m_use));
+    lsum += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+    LFrag pf;
+    pf.u = make_uint4(pack_bf16x2(e[0], e[1]), pack_bf16x2(e[2], e[3]), pack_bf16x2(e[4], e[5]),
+                      pack_bf16x2(e[6], e[7]));
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) {
+      LFrag vf;
+      vf.u2[0] = *(const uint2*)(vs + (t * 16 + r) * VS + g4 * 4);
+      vf.u2[1] = *(const uint2*)(vs + (t * 16 + r) * VS + 16 + g4 * 4);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
+    }
+  }
+  if (!row_ok) return;
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+  const float inv = 1.f / lsum;
+  bf16_t* dst = p.out + ((size_t)token * p.heads + head) * DV + g4 * 4;
+#pragma unroll
+  for (int t = 0; t < DVT; ++t)
+    *(uint2*)(dst + t * 16) = make_uint2(pack_bf16x2(acc[t][0] * inv, acc[t][1] * inv),
+                                         pack_bf16x2(acc[t][2] * inv, acc[t][3] * inv));
+}
+
 #define LATENT_MAX_PARTS 64
 
 // grid (tiles, value tiles / 4): a workgroup adds up the parts' results of 64 dims of a tile's
@@ -472,10 +646,12 @@ extern "C" int mk_attention_latent_max_parts(void) { return LATENT_MAX_PARTS; }
 
 extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache,
                                    const void* v_cache, const int* tile_seq, const int* tile_row0,
-                                   int num_tiles, const int* cu_q, const int* kv_len,
+                                   int num_tiles, int tile_rows, const int* cu_q, const int* kv_len,
                                    const int* block_table, int table_stride, int page_size,
                                    int heads, int dk, int dv, float scale, int num_parts,
                                    float* part_o, float* part_ml, hipStream_t stream) {
+  MK_REQUIRE(tile_rows == 16 || (tile_rows == 64 && num_parts == 1),
+             "latent attention: tiles of 16 rows, or of 64 with the keys unsplit");
   MK_REQUIRE(mk_attention_latent_supported(dk, dv, page_size),
              "latent attention: keys of %d, values of %d, pages of %d are not taken", dk, dv,
              page_size);
@@ -510,6 +686,15 @@ extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache
   const int waves = units >= 2048 ? LAT_WAVES : 1;
   MK_REQUIRE((units + waves - 1) / waves < (1ll << 31), "latent attention: too many tiles");
   const dim3 grid((unsigned)((units + waves - 1) / waves));
+  if (tile_rows == 64) {
+#define LATENT_STAGED(C, T)                                                \
+  if (dk == (C) * 32 && dv == (T) * 16)                                    \
+    attn_latent_staged_kernel<C, T><<<num_tiles, 256, 0, stream>>>(p);
+    LATENT_SHAPES(LATENT_STAGED)
+#undef LATENT_STAGED
+    MK_LAUNCH_CHECK("attention_latent_staged");
+    return 0;
+  }
   if (num_parts > 1 && dv == 512 && (dk == 576 || dk == 640)) {
     if (dk == 576) attn_latent_split_values_kernel<18, 32><<<(unsigned)units, 256, 0, stream>>>(p);
     else attn_latent_split_values_kernel<20, 32><<<(unsigned)units, 256, 0, stream>>>(p);

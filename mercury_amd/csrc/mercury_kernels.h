@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 24
+#define MK_ABI_VERSION 25
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
@@ -274,7 +274,9 @@ int mk_expert_down_mfma(const void* act, const void* w, float* y, const int* row
 // row f of a sequence = token f / heads, head f % heads (tile_seq / tile_row0 as for
 // mk_attention_mfma with one group of `heads`).  num_parts > 1 splits every tile's keys into
 // that many parts (at most mk_attention_latent_max_parts()) whose results part_o
-// [tiles, parts, dv, 16] / part_ml [tiles, parts, 2, 16] a second kernel merges.  No window.
+// [tiles, parts, dv, 16] / part_ml [tiles, parts, 2, 16] a second kernel merges.  tile_rows 64
+// (keys unsplit): tiles of 64 rows, one a workgroup, whose wavefronts share every block of
+// keys through LDS: for prompt portions.  No window.
 // Key and value widths come from a list of compiled shapes: mk_attention_latent_widths gives
 // the widths a cache must have for keys of at least dk and values of at least dv dims (host
 // pointers; returns 0 when no shape holds them), padded with zeros.
@@ -282,7 +284,8 @@ int mk_attention_latent_widths(int dk, int dv, int* key_width, int* value_width)
 int mk_attention_latent_supported(int dk, int dv, int page_size);
 int mk_attention_latent_max_parts(void);
 int mk_attention_latent(const void* q, void* out, const void* k_cache, const void* v_cache,
-                        const int* tile_seq, const int* tile_row0, int num_tiles, const int* cu_q,
+                        const int* tile_seq, const int* tile_row0, int num_tiles, int tile_rows,
+                        const int* cu_q,
                         const int* kv_len, const int* block_table, int table_stride, int page_size,
                         int heads, int dk, int dv, float scale, int num_parts, float* part_o,
                         float* part_ml, hipStream_t stream);

@@ -178,9 +178,10 @@ int tiles_latent_attention(const void* params, const mk_step_shape* shape, mk_ti
   view.counts = shape->counts;
   view.max_q_len = shape->max_q_len;
   view.max_kv_len = shape->max_kv_len;
-  if (!latent_plan(shape->dtype, p.latent, view).mfma) return 0;
+  const LatentPlan plan = latent_plan(shape->dtype, p.latent, view);
+  if (!plan.mfma) return 0;
   out->group = p.latent.heads;
-  out->tile_rows = 16;
+  out->tile_rows = plan.tile_rows;
   return 1;
 }
 

@@ -479,6 +479,12 @@ LatentPlan latent_plan(int dtype, const LatentArgs& a, const mk_step_view& step)
     parts = std::min(kLatentWaves / plan.num_tiles, std::max(1, blocks / kLatentMinBlocks));
   }
   plan.parts = std::max(1, std::min(parts, t.mk_attention_latent_max_parts()));
+  // Keys unsplit and some sequence with a tile of 64 rows to fill: prompt portions, whose
+  // rows share their keys through LDS.
+  if (plan.parts == 1 && (long long)step.max_q_len * a.heads >= 64) {
+    plan.tile_rows = 64;
+    plan.num_tiles = count_tiles(counts, a.heads, 64);
+  }
   return plan;
 }
 
@@ -502,9 +508,10 @@ void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scal
     part_ml = (float*)l.alloc((size_t)plan.num_tiles * plan.parts * 32 * 4);
   }
   if (l.dry() || m == 0) return out;
-  const mk_tile_list& tiles = tiles_for(step, a.heads, 16);
+  const mk_tile_list& tiles = tiles_for(step, a.heads, plan.tile_rows);
   check_mfma(need_mfma().mk_attention_latent(q.q, out, a.k_cache, a.v_cache, tiles.seq, tiles.row0,
-                                             tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride,
+                                             tiles.count, plan.tile_rows, s.cu_q, s.kv_len, s.table,
+                                             s.table_stride,
                                              a.page_size, a.heads, dk, dv, scale, plan.parts, part_o,
                                              part_ml, l.stream()), "latent_attention");
   return out;

@@ -234,6 +234,7 @@ Queries latent_queries(Launch& l, const void* x, int m, int hidden, const Latent
 struct LatentPlan {
   bool mfma = false;
   int parts = 1, num_tiles = 0;
+  int tile_rows = 16;      // 64: a workgroup's wavefronts share the keys through LDS (prompts)
 };
 LatentPlan latent_plan(int dtype, const LatentArgs& a, const mk_step_view& step);
 void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scale,

@@ -58,6 +58,7 @@ HIPCC_FLAGS = [
     "-Xclang",
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-uninitialized",
 ]
 
 
