@@ -463,3 +463,46 @@ def test_greedy_generation_through_the_engine(name):
         for i, token in enumerate(tokens):
             row = logits[len(prompt) - 1 + i]
             assert row.max() - row[token] <= 2 * BF16_SLACK * cost, f"token {i} of {tokens}"
+
+
+def test_command_line_and_sampling(tmp_path):
+    """`random-weights` and `generate` on the command line for this architecture, and sampled
+    tokens (temperature, nucleus) that do not depend on what else is in the batch."""
+    import json
+    import subprocess
+    import sys
+
+    from mercury_amd import Engine, EngineConfig, SamplingParams
+    from tests.talolorn_cases import SMALL
+
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(SMALL))
+    out = subprocess.run([sys.executable, "-m", "mercury_amd", "random-weights", "--config",
+                          str(config), "--out", str(tmp_path / "m"), "--seed", "5", "--std", "0.08"],
+                         capture_output=True, text=True, cwd=helpers.ROOT)
+    assert out.returncode == 0, out.stderr
+    prompt = [(i * 7) % 300 for i in range(20)]
+    run = subprocess.run([sys.executable, "-m", "mercury_amd", "generate", "--model",
+                          str(tmp_path / "m"), "--prompt-ids", ",".join(map(str, prompt)),
+                          "--prompt-ids", "1 2 3", "--max-tokens", "5", "--dtype", "float32",
+                          "--num-blocks", "32", "--max-model-len", "256", "--ignore-eos"],
+                         capture_output=True, text=True, cwd=helpers.ROOT)
+    assert run.returncode == 0, run.stderr
+    lines = [json.loads(line) for line in run.stdout.strip().splitlines()]
+    cfg, weights = plain.read_config(tmp_path / "m"), plain.read_weights(tmp_path / "m")
+    assert lines[0] == {"prompt_index": 0, "tokens": plain.greedy_generate(weights, cfg, prompt, 5)}
+    assert lines[1]["tokens"] == plain.greedy_generate(weights, cfg, [1, 2, 3], 5)
+
+    # a request's random numbers are keyed by the engine's seed, its id and the token's index:
+    # the first request of two engines with one seed draws the same tokens alone and in a batch
+    def fresh():
+        return Engine(EngineConfig(model=str(tmp_path / "m"), device=DEV, dtype="float32",
+                                   num_blocks=32, block_size=16, max_model_len=128, seed=9))
+
+    params = SamplingParams(temperature=0.9, top_p=0.8, ignore_eos=True)
+    others = [helpers.random_tokens(300, n, seed=n) for n in (7, 30)]
+    engine = fresh()
+    together = engine.generate([prompt] + others, params, max_tokens=10)
+    alone = fresh().generate([prompt], params, max_tokens=10)
+    assert together[0] == alone[0]
+    assert len(set(together[0])) > 1 and engine.leaked_blocks() == 0
