@@ -313,8 +313,8 @@ class TalolornConfig:
                 continue
             if not 0 <= j < len(self.layers) or self.layers[j].weights_of is not None:
                 raise ConfigError(f"layers[{i}].weights_of names {j}, which is no layer with tensors of its own")
-            if (self.layers[j].mixer, self.layers[j].mlp) != (layer.mixer, layer.mlp):
-                raise ConfigError(f"layers[{i}] uses the tensors of layer {j} but differs from it")
+            # the layer runs as layer j is described (mixer, feed-forward, norm); the rest of
+            # its own entry repeats layer j's
 
     def to_dict(self) -> dict:
         layers = []

@@ -506,3 +506,37 @@ def test_command_line_and_sampling(tmp_path):
     alone = fresh().generate([prompt], params, max_tokens=10)
     assert together[0] == alone[0]
     assert len(set(together[0])) > 1 and engine.leaked_blocks() == 0
+
+
+SHAPES = [(64, 32, 24, 16), (64, 64, 48, 16), (96, 64, 56, 16), (128, 64, 56, 48), (128, 128, 112, 16),
+          (160, 128, 120, 16), (192, 128, 120, 48), (256, 256, 240, 16), (320, 256, 248, 16),
+          (384, 256, 248, 96), (576, 512, 504, 16), (640, 512, 504, 96)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=[f"{k}x{v}" for k, v, _, _ in SHAPES])
+def test_every_compiled_cache_shape(shape, tmp_path):
+    """Latent and rotated widths that fall into each of the shapes the matrix-core attention is
+    compiled for (five heads, so tiles straddle tokens): a prompt, a portion, decoding."""
+    from mercury_amd.engine.replay import ReplaySession
+    from mercury_amd.hostcore import core
+    from mercury_amd.weights import write_random_model
+
+    key_width, value_width, kv_rank, rot = shape
+    assert core.latent_cache_widths(kv_rank + rot, kv_rank) == (key_width, value_width)
+    mixer = {"heads": 5, "dim": 16, "rot_dim": rot, "vdim": 24, "q_rank": 40, "kv_rank": kv_rank,
+             "scale": 0.2, "rot": {"base": 3000.0, "dims": rot}}
+    layer = {"type": "latent_attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": 64, "limit": 1.5}}
+    cfg = {"architecture": "Talolorn", "vocab": 257, "width": 64, "embedding": {"scale": 3.0},
+           "norm": {"eps": 1e-5}, "residual_mult": 1.3, "layers": [layer, dict(layer, weights_of=0)]}
+    folder = write_random_model(tmp_path / "m", cfg, seed=key_width + value_width, std=0.1,
+                                dtype=torch.bfloat16)
+    weights = plain.read_weights(folder)
+    tokens = helpers.random_tokens(257, 150, seed=kv_rank)
+    want = plain.forward_logits(weights, cfg, tokens)
+    cost = float((plain.forward_logits(weights, cfg, tokens, plain.to_bf16) - want).abs().max())
+    for dtype in ("float32", "bfloat16"):
+        s = ReplaySession(folder, dtype, 192)
+        rows = [s.step([entry("r", tokens[:90])], []), s.step([entry("r", tokens[90:130])], [])]
+        for i in range(130, 150):
+            rows.append(s.step([entry("r", tokens[i:i + 1])], ["r"] if i == 149 else []))
+        check(torch.cat(rows), want, dtype, f"shape {shape} {dtype}", cost)
