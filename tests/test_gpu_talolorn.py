@@ -172,19 +172,27 @@ def test_clamped_gate_feed_forward_alone(dtype, rows):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("mult", [1.0, 0.6])
-def test_parallel_block_around_the_other_mixer_and_feed_forward(dtype, mult):
+@pytest.mark.parametrize("lowered", [True, False], ids=["lowered", "from-python"])
+def test_parallel_block_around_the_other_mixer_and_feed_forward(dtype, mult, lowered):
     """The arrangement alone, with the package's ordinary attention and SiLU-gated projection as
-    its sublayers: x + m * (mixer(norm(x)) + ff(norm(x))), over two portions."""
+    its sublayers: x + m * (mixer(norm(x)) + ff(norm(x))), over two portions.  With a
+    feed-forward whose `forward` is its own (so that it cannot hand its work over) the block
+    runs from Python, on the same kernels."""
     from mercury_amd.cache import CacheManager
     from mercury_amd.engine.batch import SeqChunk, build_step
     from mercury_amd.parts import (Attention, GatedMLP, LayerCache, ParallelBlock, RMSNorm,
                                    RotaryPosition)
     from tests.plain import qwen2_plain
 
+    class OwnForward(GatedMLP):
+        def forward(self, x, step, accum):
+            return super().forward(x, step, accum)
+
     hidden, n_q, n_kv, d, page = 64, 4, 2, 16, 16
     block = ParallelBlock(Attention(hidden, n_q, n_kv, d, RotaryPosition(d, 10000.0), qkv_bias=True),
-                          GatedMLP(hidden, 96), RMSNorm(hidden, 1e-6),
+                          (GatedMLP if lowered else OwnForward)(hidden, 96), RMSNorm(hidden, 1e-6),
                           {"mixer": "attn.", "ffn": "mlp.", "norm": "norm."}, residual_mult=mult)
+    assert block.lowerable_with(None) == lowered
     params = bind_random(block, dtype, scale=0.1, seed=50)
     block.prepare(64, DEV)
     manager = CacheManager({0: block.mixer.cache_spec()}, 8, page, 2)
