@@ -524,14 +524,16 @@ SHAPES = [(64, 32, 24, 16), (64, 64, 48, 16), (96, 64, 56, 16), (128, 64, 56, 48
 @pytest.mark.parametrize("shape", SHAPES, ids=[f"{k}x{v}" for k, v, _, _ in SHAPES])
 def test_every_compiled_cache_shape(shape, tmp_path):
     """Latent and rotated widths that fall into each of the shapes the matrix-core attention is
-    compiled for (five heads, so tiles straddle tokens): a prompt, a portion, decoding."""
+    compiled for, with 5, 20, 33 or 40 heads (tiles of 16 and of 64 rows straddle tokens, or a
+    token's heads fill several tiles): a prompt, a portion, decoding."""
     from mercury_amd.engine.replay import ReplaySession
     from mercury_amd.hostcore import core
     from mercury_amd.weights import write_random_model
 
     key_width, value_width, kv_rank, rot = shape
     assert core.latent_cache_widths(kv_rank + rot, kv_rank) == (key_width, value_width)
-    mixer = {"heads": 5, "dim": 16, "rot_dim": rot, "vdim": 24, "q_rank": 40, "kv_rank": kv_rank,
+    heads = (5, 20, 33, 40)[SHAPES.index(shape) % 4]
+    mixer = {"heads": heads, "dim": 16, "rot_dim": rot, "vdim": 24, "q_rank": 40, "kv_rank": kv_rank,
              "scale": 0.2, "rot": {"base": 3000.0, "dims": rot}}
     layer = {"type": "latent_attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": 64, "limit": 1.5}}
     cfg = {"architecture": "Talolorn", "vocab": 257, "width": 64, "embedding": {"scale": 3.0},
