@@ -327,3 +327,196 @@ class TalolornConfig:
         return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
                 "embedding": {"scale": self.embedding_scale}, "norm": {"eps": self.norm_eps},
                 "residual_mult": self.residual_mult, "layers": layers}
+
+
+@dataclass(frozen=True)
+class RotatedAttentionConfig:
+    """``layers[i].mixer`` of a layer of type ``attention`` (and, with other options, the left
+    half of a ``parallel`` one): grouped-query attention whose options are all data."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot_base: float = 10000.0
+    rot_dims: int = 0            # 0: queries and keys do not turn
+    softcap: float = 0.0         # 0: the score is not bounded
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 0        # 0: no query temperature
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "RotatedAttentionConfig":
+        need = lambda key: _require_in(raw, key, where)
+        rot = raw.get("rot") or {}
+        temp = raw.get("q_temp") or {}
+        dim = int(need("dim"))
+        cfg = cls(
+            heads=int(need("heads")), kv_heads=int(need("kv_heads")), dim=dim,
+            vdim=int(raw.get("vdim", dim)), scale=float(need("scale")),
+            rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", 0)),
+            softcap=float(raw.get("softcap") or 0.0),
+            q_temp_coef=float(temp.get("coef", 0.0)), q_temp_every=int(temp.get("every", 0)))
+        for name in ("heads", "kv_heads", "dim", "vdim"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if cfg.heads % cfg.kv_heads:
+            raise ConfigError(f"{where}: {cfg.heads} heads are not a multiple of {cfg.kv_heads} kv_heads")
+        if cfg.rot_dims < 0 or cfg.rot_dims > cfg.dim or cfg.rot_dims % 2:
+            raise ConfigError(f"{where}.rot.dims {cfg.rot_dims} must be even and within dim {cfg.dim}")
+        if cfg.rot_dims and not cfg.rot_base > 0:
+            raise ConfigError(f"{where}.rot.base must be positive")
+        if cfg.softcap < 0 or cfg.q_temp_every < 0:
+            raise ConfigError(f"{where}: softcap and q_temp.every are not negative")
+        return cfg
+
+    def to_dict(self) -> dict:
+        out = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim,
+               "scale": self.scale}
+        if self.rot_dims:
+            out["rot"] = {"base": self.rot_base, "dims": self.rot_dims}
+        if self.softcap:
+            out["softcap"] = self.softcap
+        if self.q_temp_every:
+            out["q_temp"] = {"coef": self.q_temp_coef, "every": self.q_temp_every}
+        return out
+
+
+@dataclass(frozen=True)
+class StateSpaceConfig:
+    """The right half of a ``parallel`` mixer: a state-space mixer's sizes."""
+
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "StateSpaceConfig":
+        need = lambda key: int(_require_in(raw, key, where))
+        cfg = cls(heads=need("heads"), vdim=need("vdim"), state=need("state"), groups=need("groups"),
+                  conv=need("conv"), norm_groups=int(raw.get("norm_groups", 1)))
+        for name in ("heads", "vdim", "state", "groups", "conv", "norm_groups"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if cfg.heads % cfg.groups:
+            raise ConfigError(f"{where}: {cfg.heads} heads are not a multiple of {cfg.groups} groups")
+        if (cfg.heads * cfg.vdim) % cfg.norm_groups:
+            raise ConfigError(f"{where}: heads * vdim does not split into {cfg.norm_groups} norm_groups")
+        return cfg
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "vdim": self.vdim, "state": self.state, "groups": self.groups,
+                "conv": self.conv, "norm_groups": self.norm_groups}
+
+
+@dataclass(frozen=True)
+class LarozenLayerConfig:
+    kind: str                 # "attention" or "parallel"
+    attention: RotatedAttentionConfig     # the mixer, or the left half of a parallel one
+    state_space: StateSpaceConfig | None  # the right half of a parallel one
+    ff: int                   # 0: no feed-forward
+
+
+@dataclass(frozen=True)
+class LarozenConfig:
+    """The Larozen decoder: pre-norm layers (RMS norms whose stored weight lies around zero)
+    over a float32 stream; a layer's mixer is either a rotated grouped-query attention with a
+    bounded score whose values are its keys, or a sink attention and a state-space mixer side
+    by side; the feed-forward is down(relu(up(x))^2) or absent; the head is the embedding.
+    ``loop`` runs layers start .. stop - 1 `times` times in a row with the same tensors, every
+    pass over a cache and state of its own, the stream re-entering each pass through a
+    projection of itself beside the embedding output."""
+
+    vocab: int
+    width: int
+    norm_eps: float
+    layers: tuple
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1       # loop_stop == loop_start: no loop
+    architecture: str = "Larozen"
+    eos_token_ids: tuple = ()
+
+    @property
+    def loops(self) -> bool:
+        return self.loop_stop > self.loop_start
+
+    def order(self) -> list:
+        """(layer, whether the stream re-enters before it) in the order the layers run."""
+        n = len(self.layers)
+        if not self.loops:
+            return [(i, False) for i in range(n)]
+        out = [(i, False) for i in range(self.loop_start)]
+        for _ in range(self.loop_times):
+            out += [(i, i == self.loop_start) for i in range(self.loop_start, self.loop_stop)]
+        return out + [(i, False) for i in range(self.loop_stop, n)]
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "LarozenConfig":
+        entries = _require(raw, "layers")
+        if not isinstance(entries, list) or not entries:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(entries):
+            where = f"layers[{i}]"
+            kind = _require_in(entry, "type", where)
+            mixer = _require_in(entry, "mixer", where)
+            if kind == "attention":
+                attention = RotatedAttentionConfig.from_dict(mixer, where + ".mixer")
+                if attention.vdim != attention.dim:
+                    raise ConfigError(f"{where}.mixer: the values are the keys, so vdim is dim")
+                state_space = None
+            elif kind == "parallel":
+                attention = RotatedAttentionConfig.from_dict(
+                    _require_in(mixer, "left", where + ".mixer"), where + ".mixer.left")
+                state_space = StateSpaceConfig.from_dict(
+                    _require_in(mixer, "right", where + ".mixer"), where + ".mixer.right")
+            else:
+                raise ConfigError(f"{where}.type {kind!r} is not implemented; known: attention, parallel")
+            mlp = entry.get("mlp")
+            ff = 0
+            if mlp is not None:
+                if _require_in(mlp, "kind", where + ".mlp") != "dense":
+                    raise ConfigError(f"{where}.mlp.kind {mlp['kind']!r} is not implemented; known: dense")
+                ff = int(_require_in(mlp, "ff", where + ".mlp"))
+                if ff <= 0:
+                    raise ConfigError(f"{where}.mlp.ff must be positive")
+            layers.append(LarozenLayerConfig(kind, attention, state_space, ff))
+        loop = raw.get("loop") or {}
+        cfg = cls(
+            vocab=int(_require(raw, "vocab")), width=int(_require(raw, "width")),
+            norm_eps=float(_require_in(_require(raw, "norm"), "eps", "norm")),
+            layers=tuple(layers),
+            loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)) if loop else 0,
+            loop_times=int(loop.get("times", 1)),
+            architecture=str(raw.get("architecture") or (raw.get("architectures") or ["Larozen"])[0]),
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("vocab and width must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if self.loops or self.loop_times != 1:
+            if not 0 <= self.loop_start < self.loop_stop <= len(self.layers) or self.loop_times < 1:
+                raise ConfigError(f"loop: layers {self.loop_start} .. {self.loop_stop} - 1, "
+                                  f"{self.loop_times} times, of {len(self.layers)} layers")
+
+    def to_dict(self) -> dict:
+        layers = []
+        for layer in self.layers:
+            mixer = layer.attention.to_dict()
+            if layer.kind == "parallel":
+                mixer = {"left": mixer, "right": layer.state_space.to_dict()}
+            layers.append({"type": layer.kind, "mixer": mixer,
+                           "mlp": {"kind": "dense", "ff": layer.ff} if layer.ff else None})
+        out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
+               "norm": {"eps": self.norm_eps}, "layers": layers}
+        if self.loops:
+            out["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
+        return out

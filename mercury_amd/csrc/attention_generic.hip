@@ -13,6 +13,7 @@
 // Two modifications of the score the reference does not have, for mixers that want them:
 // score_cap > 0 bounds it to cap * tanh(score / cap), and distance_slopes [n_q] subtracts
 // slope[head] * (query position - key position), a position encoding that lives in the score.
+// sinks [n_q] (float32, or null): exp(sink[head]) stands in the softmax's denominator once.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -26,7 +27,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int table_stride, int page_shift, int n_q, int n_kv,
     int d, int dv, float scale, int window, float score_cap,
-    const float* __restrict__ distance_slopes) {
+    const float* __restrict__ distance_slopes, const float* __restrict__ sinks) {
   __shared__ float qs[MAXD];
   __shared__ float probs[MK_WAVE];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -88,6 +89,15 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     m = m_new;
   }
 
+  // a sink: exp(sink[head]) once more in the denominator, with no key or value behind it
+  if (sinks) {
+    const float sink = sinks[head];
+    const float m_new = fmaxf(m, sink);
+    const float corr = expf(m - m_new);
+    l = l * corr + expf(sink - m_new);
+#pragma unroll
+    for (int c = 0; c < MAXD / MK_WAVE; ++c) acc[c] *= corr;
+  }
   const float inv = 1.f / l;
 #pragma unroll
   for (int c = 0; c < MAXD / MK_WAVE; ++c) {
@@ -103,8 +113,8 @@ extern "C" int mk_attention_generic_kv(const void* q, int q_stride, void* out, i
                                        const int* positions, const int* token_seq,
                                        const int* block_table, int table_stride, int page_size,
                                        int n_q, int n_kv, int d, int dv, float scale, int window,
-                                       float score_cap, const float* distance_slopes, int tokens,
-                                       hipStream_t stream) {
+                                       float score_cap, const float* distance_slopes,
+                                       const float* sinks, int tokens, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv > 0 && d > 0 && dv > 0, "attention: bad sizes");
   MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
              n_q, n_kv);
@@ -121,7 +131,7 @@ extern "C" int mk_attention_generic_kv(const void* q, int q_stride, void* out, i
   attention_generic_kernel<T, MAXD><<<grid, MK_WAVE, 0, stream>>>(                              \
       (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_cache, (const T*)v_cache,         \
       positions, token_seq, block_table, table_stride, mk_log2(page_size), n_q, n_kv, d, dv,    \
-      scale, window, score_cap, distance_slopes)
+      scale, window, score_cap, distance_slopes, sinks)
   if (dtype == MK_F32) {
     if (widest <= AG_MAX_D) AG_LAUNCH(float, AG_MAX_D); else AG_LAUNCH(float, AG_MAX_WIDE);
   } else if (dtype == MK_BF16) {
@@ -145,5 +155,5 @@ extern "C" int mk_attention_generic(const void* q, int q_stride, void* out, int 
              AG_MAX_D);
   return mk_attention_generic_kv(q, q_stride, out, out_stride, k_cache, v_cache, dtype, positions,
                                  token_seq, block_table, table_stride, page_size, n_q, n_kv, d, d,
-                                 scale, window, score_cap, distance_slopes, tokens, stream);
+                                 scale, window, score_cap, distance_slopes, nullptr, tokens, stream);
 }

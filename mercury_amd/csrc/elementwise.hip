@@ -197,7 +197,8 @@ template <typename TO, typename TW>
 __global__ void rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ partials,
                                int num_partials, size_t partial_stride,
                                const TW* __restrict__ weight, float eps,
-                               const int* __restrict__ rows, TO* __restrict__ out, int hidden) {
+                               const int* __restrict__ rows, TO* __restrict__ out, int hidden,
+                               int once) {
   __shared__ float scratch[16];
   const int out_row = blockIdx.x;
   const int in_row = rows ? rows[out_row] : out_row;
@@ -215,7 +216,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ 
   const float rstd = rsqrtf(total / (float)hidden + eps);
   TO* dst = out + (size_t)out_row * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    const float n = Elem<TO>::round(x[i] * rstd);
+    const float n = once ? x[i] * rstd : Elem<TO>::round(x[i] * rstd);
     Elem<TO>::store(dst + i, n * Elem<TW>::load(weight + i));
   }
 }
@@ -245,7 +246,7 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ h, const float* __restric
                                    int num_partials, size_t partial_stride,
                                    const void* __restrict__ weight, float eps,
                                    const int* __restrict__ rows, TO* __restrict__ out,
-                                   int hidden) {
+                                   int hidden, int once) {
   __shared__ float scratch[16];
   const int out_row = blockIdx.x;
   const int in_row = rows ? rows[out_row] : out_row;
@@ -315,8 +316,11 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ h, const float* __restric
   for (int c = 0; c < CH; ++c) {
     const int idx = threadIdx.x + c * blockDim.x;
     if (idx >= chunks) continue;
-    const float a = Elem<TO>::round(v[c].x * rstd) * w[c].x, b = Elem<TO>::round(v[c].y * rstd) * w[c].y;
-    const float cc = Elem<TO>::round(v[c].z * rstd) * w[c].z, d = Elem<TO>::round(v[c].w * rstd) * w[c].w;
+    float a = v[c].x * rstd, b = v[c].y * rstd, cc = v[c].z * rstd, d = v[c].w * rstd;
+    if (!once) {
+      a = Elem<TO>::round(a), b = Elem<TO>::round(b), cc = Elem<TO>::round(cc), d = Elem<TO>::round(d);
+    }
+    a *= w[c].x, b *= w[c].y, cc *= w[c].z, d *= w[c].w;
     if constexpr (sizeof(TO) == 2) {
       *(uint2*)(dst + 4 * idx) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(cc, d));
     } else {
@@ -328,7 +332,7 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ h, const float* __restric
 template <typename TO>
 static int launch_rmsnorm(float* h, const float* partials, int num_partials,
                           size_t partial_stride, const void* weight, int weight_dtype, float eps,
-                          const int* rows, TO* out, int out_rows, int hidden,
+                          const int* rows, TO* out, int out_rows, int hidden, int once,
                           hipStream_t stream) {
   // Few rows (decoding): as many threads per row as it has chunks of four, so that every
   // thread waits for one group of loads only; many rows: 256 threads each.
@@ -342,10 +346,10 @@ static int launch_rmsnorm(float* h, const float* partials, int num_partials,
   do {                                                                                         \
     if (weight_dtype == MK_F32)                                                                \
       rmsnorm_vec_kernel<TO, 0, CH><<<out_rows, threads, 0, stream>>>(                         \
-          h, partials, num_partials, partial_stride, weight, eps, rows, out, hidden);          \
+          h, partials, num_partials, partial_stride, weight, eps, rows, out, hidden, once);    \
     else                                                                                       \
       rmsnorm_vec_kernel<TO, 1, CH><<<out_rows, threads, 0, stream>>>(                         \
-          h, partials, num_partials, partial_stride, weight, eps, rows, out, hidden);          \
+          h, partials, num_partials, partial_stride, weight, eps, rows, out, hidden, once);    \
     return 0;                                                                                  \
   } while (0)
     if (ch == 1) RMS_VEC(1);
@@ -358,10 +362,12 @@ static int launch_rmsnorm(float* h, const float* partials, int num_partials,
   if (out_rows <= 64 && num_partials > 0) threads = hidden >= 1024 ? 1024 : (hidden + 63) / 64 * 64;
   if (weight_dtype == MK_F32)
     rmsnorm_kernel<TO, float><<<out_rows, threads, 0, stream>>>(
-        h, partials, num_partials, partial_stride, (const float*)weight, eps, rows, out, hidden);
+        h, partials, num_partials, partial_stride, (const float*)weight, eps, rows, out, hidden,
+        once);
   else
     rmsnorm_kernel<TO, bf16_t><<<out_rows, threads, 0, stream>>>(
-        h, partials, num_partials, partial_stride, (const bf16_t*)weight, eps, rows, out, hidden);
+        h, partials, num_partials, partial_stride, (const bf16_t*)weight, eps, rows, out, hidden,
+        once);
   return 0;
 }
 
@@ -431,10 +437,10 @@ extern "C" int mk_fixed_add(long long* h64, const float* partials, int count, lo
   return 0;
 }
 
-extern "C" int mk_rmsnorm(float* h, const float* partials, int num_partials,
-                          long long partial_stride, const void* weight, int weight_dtype,
-                          float eps, const int* rows, void* out, int out_dtype, int out_rows,
-                          int hidden, hipStream_t stream) {
+extern "C" int mk_rmsnorm_rounding(float* h, const float* partials, int num_partials,
+                                   long long partial_stride, const void* weight, int weight_dtype,
+                                   float eps, const int* rows, void* out, int out_dtype,
+                                   int out_rows, int hidden, int once, hipStream_t stream) {
   MK_REQUIRE(out_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", out_rows, hidden);
   MK_REQUIRE(num_partials >= 0 && (num_partials == 0 || partials != nullptr),
              "rmsnorm: %d partial sums but no buffer", num_partials);
@@ -443,14 +449,22 @@ extern "C" int mk_rmsnorm(float* h, const float* partials, int num_partials,
   if (out_rows == 0) return 0;
   if (out_dtype == MK_F32)
     launch_rmsnorm<float>(h, partials, num_partials, (size_t)partial_stride, weight,
-                          weight_dtype, eps, rows, (float*)out, out_rows, hidden, stream);
+                          weight_dtype, eps, rows, (float*)out, out_rows, hidden, once, stream);
   else if (out_dtype == MK_BF16)
     launch_rmsnorm<bf16_t>(h, partials, num_partials, (size_t)partial_stride, weight,
-                           weight_dtype, eps, rows, (bf16_t*)out, out_rows, hidden, stream);
+                           weight_dtype, eps, rows, (bf16_t*)out, out_rows, hidden, once, stream);
   else
     MK_REQUIRE(false, "rmsnorm: unknown out dtype %d", out_dtype);
   MK_LAUNCH_CHECK("rmsnorm");
   return 0;
+}
+
+extern "C" int mk_rmsnorm(float* h, const float* partials, int num_partials,
+                          long long partial_stride, const void* weight, int weight_dtype,
+                          float eps, const int* rows, void* out, int out_dtype, int out_rows,
+                          int hidden, hipStream_t stream) {
+  return mk_rmsnorm_rounding(h, partials, num_partials, partial_stride, weight, weight_dtype, eps,
+                             rows, out, out_dtype, out_rows, hidden, 0, stream);
 }
 
 // ------------------------------------------------------------------------------ SiLU gating

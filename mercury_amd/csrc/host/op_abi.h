@@ -98,6 +98,10 @@ typedef struct mk_op_context {
   const void* out_norm_weight;
   int out_norm_weight_dtype;
   float out_norm_eps;
+  /* float32 [T, hidden] that lives for the whole step like h, for a copy of the stream an
+     operation keeps and a later one reads; there (outside a dry walk) only when a kind of the
+     program is flagged MK_OP_KEPT_STREAM */
+  float* kept;
 } mk_op_context;
 
 /* What the shape of a step is before it is packed: enough to say which tile lists an
@@ -123,8 +127,10 @@ enum {
   MK_OP_READS_X = 1,        /* needs a live x */
   MK_OP_FOLDS_PENDING = 2,  /* adds live partial sums into h; without it, live partial sums
                                before this operation are an error (they would be lost) */
-  MK_OP_FIXED_STREAM = 4    /* also works on a residual stream in fixed point (h_fixed) and
+  MK_OP_FIXED_STREAM = 4,   /* also works on a residual stream in fixed point (h_fixed) and
                                on an x left undone as a norm (norm_weight) */
+  MK_OP_KEPT_STREAM = 8     /* uses ctx->kept: a program that holds such a kind gets room for
+                               it in every step's workspace */
 };
 
 #ifdef __cplusplus

@@ -126,7 +126,11 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
                      fixed_stream(step.num_tokens);
   const size_t h_bytes = round((size_t)step.num_tokens * hidden_ * (fixed ? 8 : 4));
   const size_t logit_bytes = round((size_t)step.num_rows * vocab_ * 4);
-  const size_t persistent = own ? 0 : h_bytes + logit_bytes;
+  bool keeps = false;
+  for (const Entry& e : entries_) keeps = keeps || (e.kind.run && (e.kind.flags & MK_OP_KEPT_STREAM));
+  const size_t kept_bytes = keeps ? round((size_t)step.num_tokens * hidden_ * 4) : 0;
+  const size_t kept_at = own ? 0 : h_bytes + logit_bytes;
+  const size_t persistent = kept_at + kept_bytes;
   Arena arenas[2];
   if (dry) {
     arenas[0].reset(nullptr, 0, true);
@@ -170,6 +174,7 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
   ctx.stream_fixed = fixed ? 1 : 0;
   ctx.h_fixed = dry || !fixed ? nullptr : (long long*)workspace;
   ctx.logits = dry ? nullptr : (own ? state.own_logits : (float*)(workspace + h_bytes));
+  ctx.kept = dry || !keeps ? nullptr : (float*)(workspace + kept_at);
   ctx.alloc = &arena_alloc;
   state.h = ctx.h;
   state.logits = nullptr;

@@ -10,11 +10,13 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 25
+#define MK_ABI_VERSION 26
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
 enum { MK_ACT_SILU = 0, MK_ACT_SWISH_CLAMP = 1 };
+// Activations of one operand: the square of relu.
+enum { MK_UNARY_RELU2 = 0 };
 
 #ifdef __cplusplus
 extern "C" {
@@ -61,6 +63,13 @@ int mk_state_load(const float* state, const int* slots, const int* token_seq, vo
 int mk_rmsnorm(float* h, const float* partials, int num_partials, long long partial_stride,
                const void* weight, int weight_dtype, float eps, const int* rows, void* out,
                int out_dtype, int out_rows, int hidden, hipStream_t stream);
+
+// The same with a say in the rounding: `once` != 0 rounds x * rstd * weight once, to the
+// output type; 0 rounds the normalised value before the weight multiplies it, as mk_rmsnorm.
+int mk_rmsnorm_rounding(float* h, const float* partials, int num_partials,
+                        long long partial_stride, const void* weight, int weight_dtype, float eps,
+                        const int* rows, void* out, int out_dtype, int out_rows, int hidden,
+                        int once, hipStream_t stream);
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i].
 int mk_silu_mul(const void* gate_up, void* out, int dtype, int tokens, int inter,
@@ -109,13 +118,16 @@ int mk_fill_normal(void* out, int dtype, long long n, unsigned long long key, fl
                    float std, hipStream_t stream);
 
 // mk_attention_generic with keys of width d and values of width dv (the value cache is
-// [pages, n_kv, dv, page_size]); the output rows hold n_q heads of dv.
+// [pages, n_kv, dv, page_size]); the output rows hold n_q heads of dv.  sinks (float32 [n_q],
+// or null): exp(sink[head]) is added once to the softmax's denominator, unscaled, with no key
+// or value behind it.
 int mk_attention_generic_kv(const void* q, int q_stride, void* out, int out_stride,
                             const void* k_cache, const void* v_cache, int dtype,
                             const int* positions, const int* token_seq, const int* block_table,
                             int table_stride, int page_size, int n_q, int n_kv, int d, int dv,
                             float scale, int window, float score_cap,
-                            const float* distance_slopes, int tokens, hipStream_t stream);
+                            const float* distance_slopes, const float* sinks, int tokens,
+                            hipStream_t stream);
 
 // `batch` independent products y_b = x_b W_b^T in one launch: x_b = x + b * x_batch (rows lda
 // apart), W_b = w + b * w_batch ([N, K]), y_b = out + b * o_batch (rows ldo apart); offsets in
@@ -183,6 +195,64 @@ int mk_expert_combine(const float* pairs_out, float* y, int tokens, int top, int
 int mk_scaled_add(float* h, const float* y, const float* a, int na, const float* b, int nb,
                   long long stride, float mult, long long n, hipStream_t stream);
 int mk_fill_zero(float* p, long long n, hipStream_t stream);
+
+// Queries and keys between their projection and the cache, from a float32 row
+// [q: n_q d | k: n_kv d | v: n_kv dv] per token (the last part absent when `values_are_keys`:
+// the values are then the keys as projected, before anything below).  In this order: RMS norms
+// over the whole q part and the whole k part with weights q_norm [n_q d] and k_norm [n_kv d]
+// (both null: none); q times 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) at position p
+// (temp_every 0: none); the first `rot` dims of every head turned as in mk_rope_kv_write.
+// q goes to q_out [T, n_q d] of `dtype`, k and v into the paged cache (values [pages, n_kv, dv,
+// page_size]) when write_kv.
+int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int dtype, const void* q_norm,
+                  const void* k_norm, int norm_dtype, float eps, float temp_coef, int temp_every,
+                  const float* cos_table, const float* sin_table, int table_positions, int rot,
+                  int interleaved, const int* positions, const int* token_seq,
+                  const int* block_table, int table_stride, void* k_cache, void* v_cache,
+                  int page_size, int n_q, int n_kv, int d, int dv, int values_are_keys,
+                  int write_kv, int tokens, hipStream_t stream);
+
+// out[i] = act(x[i]) for an activation MK_UNARY_*.
+int mk_unary_act(const void* x, void* out, int dtype, long long n, int kind, hipStream_t stream);
+
+// h[t, :] += mult * (rmsnorm(a[t, :]) * wa + rmsnorm(b[t, :]) * wb), with a = ya + its `na`
+// partial sums pa[k * stride + .] (ya may be null) and b likewise (no b at all: yb null and
+// nb 0); plain weights, eps inside the root.
+int mk_normed_sum(float* h, const float* ya, const float* pa, int na, const void* wa,
+                  const float* yb, const float* pb, int nb, const void* wb, int weight_dtype,
+                  float eps, float mult, long long stride, int tokens, int hidden,
+                  hipStream_t stream);
+
+// out[t, :] = [a[t, :] | b[t, :]] in `dtype`; mk_copy_f32: dst[i] = src[i] by a kernel.
+int mk_concat_cast(const float* a, const float* b, void* out, int dtype, int tokens, int hidden,
+                   hipStream_t stream);
+int mk_copy_f32(float* dst, const float* src, long long n, hipStream_t stream);
+
+// A state-space mixer's pieces.  Per-request state lies in rows of `slot_stride` floats, a
+// sequence's row being slots[seq]; cu_q [S + 1] are the prefix sums of the step's tokens.
+// mk_causal_conv_silu: out[t, c] = silu(bias[c] + sum_j w[c, j] u_(t - taps + 1 + j)[c]) for the
+// `channels` columns of proj from col0 on, inputs before the step's first token coming from
+// `carried` ([taps - 1, channels] per slot, oldest first), which then takes the sequence's last
+// taps - 1 inputs.
+int mk_causal_conv_silu(const float* proj, int row_stride, int col0, int channels, int taps,
+                        const void* w, const void* bias, int weight_dtype, float* carried,
+                        long long slot_stride, const int* slots, const int* token_seq,
+                        const int* cu_q, float* out, int tokens, int num_seqs, hipStream_t stream);
+// mk_ssm_scan: per head S_t = exp(-exp(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T, S being N x P,
+// y_t = (S_t^T C_t + D x_t) * silu(z_t), dt_t = softplus(raw_t + dt_bias); rows of xbc are
+// [x: heads P | B: groups N | C: groups N], z and raw dt are columns z_col and dt_col of proj;
+// y_out [T, heads P].  The state is read from and written to the sequence's slot, laid out
+// as the kernel's lanes hold it: mk_ssm_state_floats says how many floats that takes (-1: sizes
+// it does not run).
+int mk_ssm_scan(const float* xbc, int xbc_stride, const float* proj, int proj_stride, int z_col,
+                int dt_col, const void* dt_bias, const void* a_log, const void* d_skip,
+                int weight_dtype, float* state, long long slot_stride, const int* slots,
+                const int* cu_q, int heads, int P, int N, int groups, float* y_out, int tokens,
+                int num_seqs, hipStream_t stream);
+long long mk_ssm_state_floats(int heads, int P, int N);
+// out[t, part] = y[t, part] / rms(y[t, part]) * weight[part], the row in `parts` equal parts.
+int mk_group_rmsnorm(const float* y, void* out, int dtype, const void* weight, int weight_dtype,
+                     float eps, int tokens, int width, int parts, hipStream_t stream);
 
 // @library mfma: bfloat16 kernels on the matrix cores
 

@@ -1,0 +1,268 @@
+// What mixers and feed-forwards of further makes need around their projections, in float32
+// arithmetic for both storage types:
+//
+//   mk_qk_prepare      queries and keys between projection and cache: norms over the whole
+//                      projection, a temperature that grows with the position, rotation of a
+//                      head's first dims, the queries out, keys and values into the paged
+//                      cache (the values may be the keys as projected);
+//   mk_unary_act       an activation of one operand (the square of relu);
+//   mk_normed_sum      h += mult * (rmsnorm(a) * wa + rmsnorm(b) * wb): mixers side by side;
+//   mk_concat_cast     [a | b] row by row, in the compute dtype (the operand of a projection
+//                      of two streams);
+//   mk_copy_f32        a copy by a kernel (a captured graph records no memcpy node here).
+#include "common.h"
+#include "mercury_kernels.h"
+
+namespace {
+
+template <typename TW>
+__device__ __forceinline__ float weight_at(const void* w, int i) {
+  return Elem<TW>::load((const TW*)w + i);
+}
+
+// One workgroup per token.  The row of qkv is [q: n_q d | k: n_kv d | v: n_kv dv], the last
+// part absent when the values are the keys.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void qk_prepare_kernel(
+    const float* __restrict__ qkv, int row_stride, T* __restrict__ q_out,
+    const void* __restrict__ q_norm, const void* __restrict__ k_norm, float eps, float temp_coef,
+    int temp_every, const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+    int rot, int interleaved, const int* __restrict__ positions,
+    const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_stride,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int page_shift, int n_q, int n_kv, int d,
+    int dv, int values_are_keys, int write_kv) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = rot / 2;
+  const float* cs = cos_table + (size_t)pos * half;
+  const float* sn = sin_table + (size_t)pos * half;
+  const float* row = qkv + (size_t)t * row_stride;
+  const int qw = n_q * d, kw = n_kv * d;
+  const float* k_src = row + qw;
+
+  float q_mult = 1.f, k_mult = 1.f;
+  if (q_norm) {
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < qw; i += blockDim.x) sq += row[i] * row[i];
+    q_mult = rsqrtf(block_sum(sq, scratch) / (float)qw + eps);
+  }
+  if (k_norm && write_kv) {
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < kw; i += blockDim.x) sq += k_src[i] * k_src[i];
+    k_mult = rsqrtf(block_sum(sq, scratch) / (float)kw + eps);
+  }
+  if (temp_every > 0) {
+    q_mult *= 1.f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.f);
+  }
+
+  // the value of entry i of q (of k) before it turns
+  auto q_at = [&](int i) {
+    const float v = row[i] * q_mult;
+    return q_norm ? v * weight_at<TW>(q_norm, i) : v;
+  };
+  auto k_at = [&](int i) {
+    const float v = k_src[i] * k_mult;
+    return k_norm ? v * weight_at<TW>(k_norm, i) : v;
+  };
+  // entry j of a head after the turn: the partner is j ^ 1 (interleaved) or j -+ half
+  auto turned = [&](auto at, int base, int j) {
+    if (j >= rot) return at(base + j);
+    if (interleaved) {
+      const int pair = j >> 1;
+      return (j & 1) ? at(base + j) * cs[pair] + at(base + j - 1) * sn[pair]
+                     : at(base + j) * cs[pair] - at(base + j + 1) * sn[pair];
+    }
+    return j < half ? at(base + j) * cs[j] - at(base + j + half) * sn[j]
+                    : at(base + j) * cs[j - half] + at(base + j - half) * sn[j - half];
+  };
+
+  for (int i = threadIdx.x; i < qw; i += blockDim.x) {
+    const int head = i / d, j = i - head * d;
+    Elem<T>::store(q_out + (size_t)t * qw + i, turned(q_at, head * d, j));
+  }
+  if (!write_kv) return;
+
+  const int page_size = 1 << page_shift;
+  const int page = block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)];
+  if (page < 0) return;  // the host never schedules a write into a page that was given back
+  const int off = pos & (page_size - 1);
+  for (int i = threadIdx.x; i < kw; i += blockDim.x) {
+    const int head = i / d, j = i - head * d;
+    const size_t dst = (((size_t)page * n_kv + head) * page_size + off) * d + j;
+    Elem<T>::store(k_cache + dst, turned(k_at, head * d, j));
+  }
+  const float* v_src = values_are_keys ? k_src : k_src + kw;
+  for (int i = threadIdx.x; i < n_kv * dv; i += blockDim.x) {
+    const int head = i / dv, j = i - head * dv;
+    Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * dv + j) * page_size + off, v_src[i]);
+  }
+}
+
+template <typename T>
+__global__ void unary_act_kernel(const T* __restrict__ x, T* __restrict__ out, long long n,
+                                 int kind) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = Elem<T>::load(x + i);
+  float y = v;
+  if (kind == MK_UNARY_RELU2) {
+    const float r = fmaxf(v, 0.f);
+    y = r * r;
+  }
+  Elem<T>::store(out + i, y);
+}
+
+// One workgroup per token: the two rows' sums of squares, then the weighted sum.
+template <typename TW>
+__global__ __launch_bounds__(256) void normed_sum_kernel(
+    float* __restrict__ h, const float* __restrict__ ya, const float* __restrict__ pa, int na,
+    const void* __restrict__ wa, const float* __restrict__ yb, const float* __restrict__ pb,
+    int nb, const void* __restrict__ wb, float eps, float mult, size_t stride, int hidden) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * hidden;
+  auto value = [&](const float* y, const float* p, int n, int i) {
+    float v = y ? y[base + i] : 0.f;
+    for (int k = 0; k < n; ++k) v += p[(size_t)k * stride + base + i];
+    return v;
+  };
+  const bool has_b = yb != nullptr || nb > 0;
+  float sa = 0.f, sb = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float a = value(ya, pa, na, i);
+    sa += a * a;
+    if (has_b) {
+      const float b = value(yb, pb, nb, i);
+      sb += b * b;
+    }
+  }
+  const float ra = rsqrtf(block_sum(sa, scratch) / (float)hidden + eps);
+  const float rb = has_b ? rsqrtf(block_sum(sb, scratch) / (float)hidden + eps) : 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float sum = value(ya, pa, na, i) * ra * weight_at<TW>(wa, i);
+    if (has_b) sum += value(yb, pb, nb, i) * rb * weight_at<TW>(wb, i);
+    h[base + i] += mult * sum;
+  }
+}
+
+template <typename T>
+__global__ void concat_cast_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                   T* __restrict__ out, int hidden) {
+  const size_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    Elem<T>::store(out + t * 2 * hidden + i, a[t * hidden + i]);
+    Elem<T>::store(out + t * 2 * hidden + hidden + i, b[t * hidden + i]);
+  }
+}
+
+__global__ void copy_f32_kernel(float* __restrict__ dst, const float* __restrict__ src,
+                                long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+}  // namespace
+
+extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int dtype,
+                             const void* q_norm, const void* k_norm, int norm_dtype, float eps,
+                             float temp_coef, int temp_every, const float* cos_table,
+                             const float* sin_table, int table_positions, int rot,
+                             int interleaved, const int* positions, const int* token_seq,
+                             const int* block_table, int table_stride, void* k_cache,
+                             void* v_cache, int page_size, int n_q, int n_kv, int d, int dv,
+                             int values_are_keys, int write_kv, int tokens, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv >= 0 && d > 0 && dv > 0, "qk_prepare: bad sizes");
+  MK_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0,
+             "qk_prepare: rotary width %d not in [0, %d] / even", rot, d);
+  MK_REQUIRE(rot == 0 || (table_positions > 0 && cos_table && sin_table),
+             "qk_prepare: empty angle table");
+  MK_REQUIRE(mk_is_pow2(page_size), "qk_prepare: page size %d is not a power of two", page_size);
+  MK_REQUIRE(!values_are_keys || dv == d, "qk_prepare: values that are keys are as wide as keys");
+  const int need = n_q * d + (write_kv ? n_kv * d + (values_are_keys ? 0 : n_kv * dv) : 0);
+  MK_REQUIRE(row_stride >= need, "qk_prepare: row stride %d below the %d columns of q, k, v",
+             row_stride, need);
+  MK_REQUIRE((q_norm == nullptr) == (k_norm == nullptr) || !write_kv,
+             "qk_prepare: a norm for queries and keys alike");
+  MK_REQUIRE(temp_every >= 0, "qk_prepare: negative temperature period");
+  MK_REQUIRE(!write_kv || (k_cache && v_cache && block_table), "qk_prepare: no cache to write");
+  MK_REQUIRE(norm_dtype == MK_F32 || norm_dtype == MK_BF16, "qk_prepare: norm dtype %d", norm_dtype);
+  if (tokens == 0) return 0;
+#define QK_LAUNCH(T, TW)                                                                         \
+  qk_prepare_kernel<T, TW><<<tokens, 256, 0, stream>>>(                                          \
+      qkv, row_stride, (T*)q_out, q_norm, k_norm, eps, temp_coef, temp_every, cos_table,         \
+      sin_table, rot, interleaved, positions, token_seq, block_table, table_stride, (T*)k_cache, \
+      (T*)v_cache, mk_log2(page_size), n_q, n_kv, d, dv, values_are_keys, write_kv)
+  if (dtype == MK_F32) {
+    if (norm_dtype == MK_F32) QK_LAUNCH(float, float); else QK_LAUNCH(float, bf16_t);
+  } else if (dtype == MK_BF16) {
+    if (norm_dtype == MK_F32) QK_LAUNCH(bf16_t, float); else QK_LAUNCH(bf16_t, bf16_t);
+  } else {
+    MK_REQUIRE(false, "qk_prepare: unknown dtype %d", dtype);
+  }
+#undef QK_LAUNCH
+  MK_LAUNCH_CHECK("qk_prepare");
+  return 0;
+}
+
+extern "C" int mk_unary_act(const void* x, void* out, int dtype, long long n, int kind,
+                            hipStream_t stream) {
+  MK_REQUIRE(n >= 0, "unary_act: negative count");
+  MK_REQUIRE(kind == MK_UNARY_RELU2, "unary_act: unknown activation %d", kind);
+  if (n == 0) return 0;
+  const long long blocks = (n + 255) / 256;
+  MK_REQUIRE(blocks < (1ll << 31), "unary_act: %lld elements are too many for one launch", n);
+  if (dtype == MK_F32)
+    unary_act_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)x, (float*)out, n, kind);
+  else if (dtype == MK_BF16)
+    unary_act_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, n, kind);
+  else
+    MK_REQUIRE(false, "unary_act: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("unary_act");
+  return 0;
+}
+
+extern "C" int mk_normed_sum(float* h, const float* ya, const float* pa, int na, const void* wa,
+                             const float* yb, const float* pb, int nb, const void* wb,
+                             int weight_dtype, float eps, float mult, long long stride, int tokens,
+                             int hidden, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && hidden > 0, "normed_sum: bad sizes");
+  MK_REQUIRE(na >= 0 && nb >= 0 && (na == 0 || pa) && (nb == 0 || pb),
+             "normed_sum: partial sums without a buffer");
+  MK_REQUIRE((ya || na) && wa, "normed_sum: no first operand");
+  MK_REQUIRE(!(yb || nb) || wb, "normed_sum: a second operand without its weight");
+  MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "normed_sum: weight dtype %d",
+             weight_dtype);
+  if (tokens == 0) return 0;
+  if (weight_dtype == MK_F32)
+    normed_sum_kernel<float><<<tokens, 256, 0, stream>>>(h, ya, pa, na, wa, yb, pb, nb, wb, eps,
+                                                          mult, (size_t)stride, hidden);
+  else
+    normed_sum_kernel<bf16_t><<<tokens, 256, 0, stream>>>(h, ya, pa, na, wa, yb, pb, nb, wb, eps,
+                                                           mult, (size_t)stride, hidden);
+  MK_LAUNCH_CHECK("normed_sum");
+  return 0;
+}
+
+extern "C" int mk_concat_cast(const float* a, const float* b, void* out, int dtype, int tokens,
+                              int hidden, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && hidden > 0, "concat_cast: bad sizes");
+  if (tokens == 0) return 0;
+  if (dtype == MK_F32)
+    concat_cast_kernel<float><<<tokens, 256, 0, stream>>>(a, b, (float*)out, hidden);
+  else if (dtype == MK_BF16)
+    concat_cast_kernel<bf16_t><<<tokens, 256, 0, stream>>>(a, b, (bf16_t*)out, hidden);
+  else
+    MK_REQUIRE(false, "concat_cast: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("concat_cast");
+  return 0;
+}
+
+extern "C" int mk_copy_f32(float* dst, const float* src, long long n, hipStream_t stream) {
+  MK_REQUIRE(n >= 0, "copy: negative count");
+  if (n == 0) return 0;
+  const long long blocks = (n + 255) / 256;
+  MK_REQUIRE(blocks < (1ll << 31), "copy: %lld elements are too many for one launch", n);
+  copy_f32_kernel<<<(unsigned)blocks, 256, 0, stream>>>(dst, src, n);
+  MK_LAUNCH_CHECK("copy");
+  return 0;
+}

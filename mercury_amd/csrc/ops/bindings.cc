@@ -208,14 +208,17 @@ void bind_ops(py::module_& m) {
     p.scale = scale;
     return blob(p);
   }, py::arg("table"), py::arg("table_dtype"), py::arg("vocab"), py::arg("scale") = 1.f);
-  m.def("norm_params", [](uintptr_t weight, int weight_dtype, float eps, bool select_rows) {
+  m.def("norm_params", [](uintptr_t weight, int weight_dtype, float eps, bool select_rows,
+                           bool round_once) {
     NormParams p;
     p.weight = as_ptr<const void>(weight);
     p.weight_dtype = weight_dtype;
     p.eps = eps;
     p.select_rows = select_rows ? 1 : 0;
+    p.round_once = round_once ? 1 : 0;
     return blob(p);
-  }, py::arg("weight"), py::arg("weight_dtype"), py::arg("eps"), py::arg("select_rows") = false);
+  }, py::arg("weight"), py::arg("weight_dtype"), py::arg("eps"), py::arg("select_rows") = false,
+     py::arg("round_once") = false);
   m.def("attention_params", [](const py::kwargs& kw) {
     const py::dict d = kw;
     AttentionParams p;
@@ -228,8 +231,101 @@ void bind_ops(py::module_& m) {
     p.scale = get<float>(d, "scale", 0.f);
     p.score_cap = get<float>(d, "score_cap", 0.f);
     p.distance_slopes = ptr_of<const float>(d, "distance_slopes");
+    p.sinks = ptr_of<const float>(d, "sinks");
+    p.prep.q_norm = ptr_of<const void>(d, "q_norm");
+    p.prep.k_norm = ptr_of<const void>(d, "k_norm");
+    p.prep.norm_dtype = get<int>(d, "norm_dtype", kF32);
+    p.prep.eps = get<float>(d, "norm_eps", 0.f);
+    p.prep.temp_coef = get<float>(d, "temp_coef", 0.f);
+    p.prep.temp_every = get<int>(d, "temp_every", 0);
+    p.prep.values_are_keys = get<bool>(d, "values_are_keys", false) ? 1 : 0;
+    p.prep.value_dim = get<int>(d, "value_dim", 0);
+    if ((p.prep.q_norm == nullptr) != (p.prep.k_norm == nullptr)) {
+      throw KernelError("attention: a norm for queries and keys alike");
+    }
+    if (p.prep.temp_every < 0) throw KernelError("attention: negative temperature period");
+    if (p.prep.values_are_keys && p.prep.value_dim > 0 && p.prep.value_dim != p.qkv.head_dim) {
+      throw KernelError("attention: values that are keys are as wide as keys");
+    }
     return blob(p);
   });
+  m.def("unary_mlp_params", [](uintptr_t w_up, uintptr_t w_down, int inter, int act) {
+    if (act != MK_UNARY_RELU2) throw KernelError("unknown activation " + std::to_string(act));
+    UnaryMlpParams p;
+    p.w_up = as_ptr<const void>(w_up);
+    p.w_down = as_ptr<const void>(w_down);
+    p.inter = inter;
+    p.act = act;
+    return blob(p);
+  }, py::arg("w_up"), py::arg("w_down"), py::arg("inter"), py::arg("act") = 0);
+  m.def("ssm_state_floats", [](int heads, int vdim, int state_size) {
+    const long long n = need_core().mk_ssm_state_floats(heads, vdim, state_size);
+    if (n < 0) throw KernelError("state_space: the recurrence does not run these sizes");
+    return n;
+  }, "Floats of recurrent state a request holds for `heads` heads of [state_size, vdim].");
+  m.def("state_space_params", [](const py::kwargs& kw) {
+    const py::dict d = kw;
+    StateSpaceParams p;
+    StateSpaceArgs& a = p.args;
+    a.w_in = ptr_of<const void>(d, "w_in");
+    a.conv_w = ptr_of<const void>(d, "conv_w");
+    a.conv_b = ptr_of<const void>(d, "conv_b");
+    a.dt_bias = ptr_of<const void>(d, "dt_bias");
+    a.a_log = ptr_of<const void>(d, "a_log");
+    a.d_skip = ptr_of<const void>(d, "d_skip");
+    a.norm = ptr_of<const void>(d, "norm");
+    a.vector_dtype = get<int>(d, "vector_dtype", kF32);
+    a.w_out = ptr_of<const void>(d, "w_out");
+    a.heads = get<int>(d, "heads", 0);
+    a.vdim = get<int>(d, "vdim", 0);
+    a.state_size = get<int>(d, "state_size", 0);
+    a.groups = get<int>(d, "groups", 0);
+    a.taps = get<int>(d, "taps", 0);
+    a.norm_groups = get<int>(d, "norm_groups", 1);
+    a.eps = get<float>(d, "eps", 0.f);
+    a.state = ptr_of<float>(d, "state");
+    a.slot_floats = get<long long>(d, "slot_floats", 0);
+    if (a.heads <= 0 || a.vdim <= 0 || a.state_size <= 0 || a.groups <= 0 || a.taps < 1 ||
+        a.norm_groups <= 0 || a.heads % a.groups || a.inner() % a.norm_groups) {
+      throw KernelError("state_space: bad sizes");
+    }
+    return blob(p);
+  });
+  m.def("normed_sum_params", [](float mult, float eps, int weight_dtype,
+                                 const std::vector<std::tuple<std::string, py::bytes, uintptr_t>>& subs) {
+    if (subs.empty() || (int)subs.size() > kNormedSumMax) {
+      throw KernelError("a normed sum holds 1 to " + std::to_string(kNormedSumMax) + " sublayers");
+    }
+    NormedSumParams p;
+    p.mult = mult;
+    p.eps = eps;
+    p.weight_dtype = weight_dtype;
+    p.count = (int)subs.size();
+    std::string out(sizeof p, '\0');
+    for (size_t i = 0; i < subs.size(); ++i) {
+      const OpKind& kind = OpRegistry::instance().get(std::get<0>(subs[i]));
+      if (kind.flags & MK_OP_FOLDS_PENDING) {
+        throw KernelError("a sublayer of a normed sum cannot be an operation that adds up partial sums");
+      }
+      const std::string bytes = std::get<1>(subs[i]);
+      out.resize((out.size() + 15) / 16 * 16, '\0');
+      p.sub[i].run = kind.run;
+      p.sub[i].tiles = kind.tiles;
+      p.sub[i].flags = kind.flags;
+      p.sub[i].offset = (int)out.size();
+      p.sub[i].weight = as_ptr<const void>(std::get<2>(subs[i]));
+      out += bytes;
+    }
+    std::memcpy(&out[0], &p, sizeof p);
+    return py::bytes(out);
+  }, py::arg("mult"), py::arg("eps"), py::arg("weight_dtype"), py::arg("sublayers"),
+     "The parameter block of a 'normed_sum' operation: sublayers as (kind, parameter bytes, "
+     "address of the weight of the norm over its output).");
+  m.def("stream_mix_params", [](uintptr_t weight) {
+    StreamMixParams p;
+    p.weight = as_ptr<const void>(weight);
+    return blob(p);
+  }, py::arg("weight"));
   m.def("gated_mlp_params", [](uintptr_t w_gate_up, uintptr_t w_down, int inter, int act,
                                 float limit, float alpha, float beta) {
     GatedMlpParams p;

@@ -84,7 +84,7 @@ int run_norm(const void* params, mk_op_context* ctx) {
     }
     ctx->out_x = rmsnorm(l, ctx->h, s.num_tokens, ctx->hidden, ctx->pending, ctx->pending_count,
                          p.weight, p.weight_dtype, p.eps, p.select_rows ? s.logit_rows : nullptr,
-                         rows);
+                         rows, nullptr, p.round_once != 0);
     ctx->out_x_rows = rows;
     ctx->out_x_live = 1;
   });
@@ -102,6 +102,8 @@ AttendArgs attend_args(const AttentionParams& p) {
   a.v_cache = p.qkv.v_cache;
   a.score_cap = p.score_cap;
   a.distance_slopes = p.distance_slopes;
+  a.sinks = p.sinks;
+  a.value_dim = p.prep.value_dim;
   return a;
 }
 
@@ -113,8 +115,13 @@ int run_attention(const void* params, mk_op_context* ctx) {
     Launch l(ctx);
     const StepArrays arrays = arrays_of(s, p.group);
     NormFold fold;
-    const Queries q = qkv_project(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, arrays, {},
-                                  fold_of(ctx, fold));
+    if (p.prep.active() && ctx->stream_fixed) {
+      throw KernelError("attention: norms over q and k, a query temperature or values that are "
+                        "keys do not run on a stream in fixed point");
+    }
+    const Queries q = p.prep.active()
+        ? qkv_prepared(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, p.prep, arrays)
+        : qkv_project(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, arrays, {}, fold_of(ctx, fold));
     attend_and_project(l, q, attend_args(p), arrays, s, p.w_o, p.b_o, p.b_o_dtype, ctx->hidden,
                        ctx->h, ctx->out_pending, ctx->out_pending_count, {}, -1, ctx->h_fixed);
   });
@@ -192,6 +199,100 @@ int run_routed_experts(const void* params, mk_op_context* ctx) {
     if (ctx->x_rows != m) throw KernelError("the experts read an x of every token");
     Launch l(ctx);
     routed_experts(l, ctx->x, m, ctx->hidden, p.experts, ctx->h);
+  });
+}
+
+int run_unary_mlp(const void* params, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    const UnaryMlpParams& p = *static_cast<const UnaryMlpParams*>(params);
+    const int m = ctx->step->num_tokens;
+    if (ctx->x_rows != m) throw KernelError("the feed-forward reads an x of every token");
+    Launch l(ctx);
+    unary_mlp(l, ctx->x, m, ctx->hidden, p.w_up, p.w_down, p.inter, p.act, ctx->h,
+              ctx->out_pending, ctx->out_pending_count);
+  });
+}
+
+int run_state_space(const void* params, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    const StateSpaceParams& p = *static_cast<const StateSpaceParams*>(params);
+    const mk_step_view& s = *ctx->step;
+    if (ctx->x_rows != s.num_tokens) throw KernelError("the mixer reads an x of every token");
+    Launch l(ctx);
+    state_space(l, ctx->x, s.num_tokens, ctx->hidden, p.args, s, ctx->h, ctx->out_pending,
+                ctx->out_pending_count);
+  });
+}
+
+// Every sublayer adds into a zeroed buffer of its own in the stream's place; what it leaves as
+// partial sums is added to that buffer inside the kernel that norms and sums.
+int run_normed_sum(const void* params, mk_op_context* ctx) {
+  const NormedSumParams& p = *static_cast<const NormedSumParams*>(params);
+  const int tokens = ctx->step->num_tokens;
+  const long long n = (long long)tokens * ctx->hidden;
+  float* const h = ctx->h;
+  float* y[kNormedSumMax] = {nullptr};
+  const float* parts[kNormedSumMax] = {nullptr};
+  int counts[kNormedSumMax] = {0};
+  if (p.count < 1 || p.count > kNormedSumMax) {
+    std::snprintf(ctx->error, sizeof ctx->error, "normed_sum: %d sublayers", p.count);
+    return 1;
+  }
+  for (int i = 0; i < p.count; ++i) {
+    const int code = guarded(ctx, [&] {
+      Launch l(ctx);
+      y[i] = zeros(l, n);
+    });
+    if (code) return code;
+    ctx->h = y[i];
+    ctx->out_x = nullptr;
+    ctx->out_x_rows = ctx->out_x_live = 0;
+    ctx->out_pending = nullptr;
+    ctx->out_pending_count = 0;
+    const int ran = p.sub[i].run(static_cast<const char*>(params) + p.sub[i].offset, ctx);
+    ctx->h = h;
+    if (ran) return ran;
+    parts[i] = ctx->out_pending;
+    counts[i] = ctx->out_pending_count;
+  }
+  ctx->out_x = nullptr;
+  ctx->out_x_rows = ctx->out_x_live = 0;
+  ctx->out_pending = nullptr;
+  ctx->out_pending_count = 0;
+  ctx->out_logits_ready = 0;
+  return guarded(ctx, [&] {
+    Launch l(ctx);
+    normed_sum(l, h, y[0], parts[0], counts[0], p.sub[0].weight, p.count > 1 ? y[1] : nullptr,
+               parts[1], counts[1], p.count > 1 ? p.sub[1].weight : nullptr, p.weight_dtype, p.eps,
+               p.mult, tokens, ctx->hidden);
+  });
+}
+
+int tiles_normed_sum(const void* params, const mk_step_shape* shape, mk_tile_need* out) {
+  const NormedSumParams& p = *static_cast<const NormedSumParams*>(params);
+  for (int i = 0; i < p.count; ++i) {
+    if (p.sub[i].tiles &&
+        p.sub[i].tiles(static_cast<const char*>(params) + p.sub[i].offset, shape, out) > 0) {
+      return 1;
+    }
+  }
+  return 0;
+}
+
+int run_keep_stream(const void*, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    Launch l(ctx);
+    if (!l.dry() && !ctx->kept) throw KernelError("keep_stream: the step has no room to keep a stream");
+    copy_stream(l, ctx->kept, ctx->h, (long long)ctx->step->num_tokens * ctx->hidden);
+  });
+}
+
+int run_stream_mix(const void* params, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    const StreamMixParams& p = *static_cast<const StreamMixParams*>(params);
+    Launch l(ctx);
+    if (!l.dry() && !ctx->kept) throw KernelError("stream_mix: no stream was kept in this step");
+    stream_mix(l, ctx->h, ctx->kept, ctx->step->num_tokens, ctx->hidden, p.weight);
   });
 }
 
@@ -288,6 +389,11 @@ void register_builtin_ops() {
   r.add(OpKind{"latent_attention", &run_latent_attention, &tiles_latent_attention, MK_OP_READS_X});
   r.add(OpKind{"routed_experts", &run_routed_experts, nullptr, MK_OP_READS_X});
   r.add(OpKind{"parallel", &run_parallel, &tiles_parallel, MK_OP_READS_X});
+  r.add(OpKind{"unary_mlp", &run_unary_mlp, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"state_space", &run_state_space, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"normed_sum", &run_normed_sum, &tiles_normed_sum, MK_OP_READS_X});
+  r.add(OpKind{"keep_stream", &run_keep_stream, nullptr, MK_OP_KEPT_STREAM});
+  r.add(OpKind{"stream_mix", &run_stream_mix, nullptr, MK_OP_KEPT_STREAM});
   r.add(OpKind{"head", &run_head, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
   r.fixed_stream_tokens = &fixed_stream_tokens;
 }

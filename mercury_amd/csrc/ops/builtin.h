@@ -21,6 +21,7 @@ struct NormParams {
   int weight_dtype = 0;
   float eps = 0.f;
   int select_rows = 0;
+  int round_once = 0;     // x * rstd * weight rounded once, not the normalised value first
 };
 
 // "attention": q/k/v projection, position encoding, cache write, softmax attention over the
@@ -34,6 +35,44 @@ struct AttentionParams {
   float scale = 0.f;
   float score_cap = 0.f;                    // > 0: the score is bounded to cap * tanh(. / cap)
   const float* distance_slopes = nullptr;   // [n_q]: slope * distance is subtracted from it
+  const float* sinks = nullptr;             // [n_q]: exp(sink) once more in the denominator
+  QkPrep prep;                              // norms over q and k, query temperature, v = k
+};
+
+// "unary_mlp": h += act(x Wu^T) Wd^T for an activation of one operand (or left as partial sums).
+struct UnaryMlpParams {
+  const void *w_up = nullptr, *w_down = nullptr;
+  int inter = 0;
+  int act = 0;
+};
+
+// "state_space": a state-space mixer over per-request state (launch.h), its output projection
+// into h (or left as partial sums).
+struct StateSpaceParams {
+  StateSpaceArgs args;
+};
+
+// "normed_sum": mixers side by side on the same x; each one's output is RMS-normed over the
+// model width with a plain weight of its own, and h += mult * their sum.  Laid out as
+// "parallel": this header, then the sublayers' parameter blocks at `offset`.
+constexpr int kNormedSumMax = 2;
+struct NormedSumParams {
+  float mult = 1.f, eps = 0.f;
+  int count = 0;
+  int weight_dtype = 0;
+  struct Sub {
+    mk_op_run_fn run = nullptr;
+    mk_op_tiles_fn tiles = nullptr;
+    int flags = 0;
+    int offset = 0;
+    const void* weight = nullptr;
+  } sub[kNormedSumMax];
+};
+
+// "keep_stream": the residual stream as it stands is kept for the rest of the step.
+// "stream_mix": h <- [h | kept] W^T, W [hidden, 2 hidden].
+struct StreamMixParams {
+  const void* weight = nullptr;
 };
 
 // "gated_mlp": h += (act(x Wg^T) * (x Wu^T)) Wd^T (or left as partial sums).

@@ -17,12 +17,13 @@ void embed(Launch& l, const int* ids, const void* table, int table_dtype, float*
 
 void* rmsnorm(Launch& l, float* h, int tokens, int hidden, const float* pending, int pending_count,
               const void* weight, int weight_dtype, float eps, const int* rows, int out_rows,
-              void* out) {
+              void* out, bool round_once) {
   if (!out) out = l.alloc((size_t)out_rows * hidden * l.elem());
   if (l.dry() || out_rows == 0) return out;
-  check_core(need_core().mk_rmsnorm(h, pending, pending_count, (long long)tokens * hidden, weight,
-                                    weight_dtype, eps, rows, out, l.dtype(), out_rows, hidden,
-                                    l.stream()), "rmsnorm");
+  check_core(need_core().mk_rmsnorm_rounding(h, pending, pending_count, (long long)tokens * hidden,
+                                             weight, weight_dtype, eps, rows, out, l.dtype(),
+                                             out_rows, hidden, round_once ? 1 : 0, l.stream()),
+             "rmsnorm");
   return out;
 }
 
@@ -239,6 +240,26 @@ Queries qkv_project(Launch& l, const void* x, int m, int k, const QkvArgs& a, co
   return {qkv, width};
 }
 
+Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, const QkPrep& prep,
+                     const StepArrays& s) {
+  const int d = a.head_dim, dv = prep.value_dim > 0 ? prep.value_dim : d;
+  const int heads_kv = kv_heads(a);
+  const int width = a.n_q * d + heads_kv * d + (prep.values_are_keys ? 0 : heads_kv * dv);
+  const float* qkv = (const float*)linear(l, x, m, a.w, width, k, a.bias,
+                                          a.bias ? a.bias_dtype : kF32, nullptr, kF32, false);
+  void* q = l.alloc((size_t)m * a.n_q * d * l.elem());
+  if (l.dry() || m == 0) return {q, a.n_q * d};
+  const PositionDesc& p = a.pos;
+  check_core(need_core().mk_qk_prepare(
+                 qkv, width, q, l.dtype(), prep.q_norm, prep.k_norm, prep.norm_dtype, prep.eps,
+                 prep.temp_coef, prep.temp_every, p.cos, p.sin, p.table_positions, p.rotary_dim,
+                 p.interleaved ? 1 : 0, s.positions, s.token_seq, s.table, s.table_stride,
+                 a.writes ? a.k_cache : nullptr, a.writes ? a.v_cache : nullptr,
+                 a.writes ? a.page_size : 1, a.n_q, heads_kv, d, dv, prep.values_are_keys,
+                 a.writes ? 1 : 0, m, l.stream()), "qk_prepare");
+  return {q, a.n_q * d};
+}
+
 AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
                        const AttendForce& force) {
   if (!a.plain_scores()) {
@@ -280,7 +301,7 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
       check_core(need_core().mk_attention_generic_kv(
                      q.q, q.stride, out, a.n_q * a.v_dim(), a.k_cache, a.v_cache, l.dtype(),
                      s.positions, s.token_seq, s.table, s.table_stride, a.page_size, a.n_q, a.n_kv,
-                     d, a.v_dim(), a.scale, a.window, a.score_cap, a.distance_slopes, m,
+                     d, a.v_dim(), a.scale, a.window, a.score_cap, a.distance_slopes, a.sinks, m,
                      l.stream()), "attention");
     }
     return out;
@@ -342,10 +363,10 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
     if (fold > 0) throw KernelError("attention: these sizes do not take the folded merge");
     const void* attended = attend(l, q, a, s, step, force);
     if (fixed) {
-      project_into_fixed(l, attended, m, w_o, hidden, a.n_q * d, b_o, b_o_dtype, h_fixed);
+      project_into_fixed(l, attended, m, w_o, hidden, a.n_q * a.v_dim(), b_o, b_o_dtype, h_fixed);
     } else {
-      project_into_stream(l, attended, m, w_o, hidden, a.n_q * d, b_o, b_o_dtype, h, pending,
-                          pending_count);
+      project_into_stream(l, attended, m, w_o, hidden, a.n_q * a.v_dim(), b_o, b_o_dtype, h,
+                          pending, pending_count);
     }
     return;
   }
@@ -402,6 +423,70 @@ void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int i
   if (tile_config != -2) throw KernelError("gated_projection: operands not eligible");
   void* gate_up = linear(l, x, m, w_gate_up, 2 * inter, k, nullptr, kF32, nullptr, l.dtype(), false);
   return act.silu() ? silu_mul(l, gate_up, m, inter) : gate_activation(l, gate_up, m, inter, act);
+}
+
+void unary_mlp(Launch& l, const void* x, int m, int hidden, const void* w_up, const void* w_down,
+               int inter, int act, float* h, const float*& pending, int& pending_count) {
+  pending = nullptr;
+  pending_count = 0;
+  void* up = linear(l, x, m, w_up, inter, hidden, nullptr, kF32, nullptr, l.dtype(), false);
+  void* acted = l.alloc((size_t)m * inter * l.elem());
+  if (!l.dry() && m > 0) {
+    check_core(need_core().mk_unary_act(up, acted, l.dtype(), (long long)m * inter, act,
+                                        l.stream()), "unary_act");
+  }
+  project_into_stream(l, acted, m, w_down, hidden, inter, nullptr, kF32, h, pending,
+                      pending_count);
+}
+
+void state_space(Launch& l, const void* x, int m, int hidden, const StateSpaceArgs& a,
+                 const mk_step_view& step, float* h, const float*& pending, int& pending_count) {
+  pending = nullptr;
+  pending_count = 0;
+  const int inner = a.inner(), channels = a.channels(), width = a.in_width();
+  const float* proj = (const float*)linear(l, x, m, a.w_in, width, hidden, nullptr, kF32, nullptr,
+                                           kF32, false);
+  float* xbc = (float*)l.alloc((size_t)m * channels * 4);
+  float* y = (float*)l.alloc((size_t)m * inner * 4);
+  void* normed = l.alloc((size_t)m * inner * l.elem());
+  if (!l.dry() && m > 0) {
+    const KernelTable& t = need_core();
+    if (!a.state) throw KernelError("state_space: no state tensor");
+    check_core(t.mk_causal_conv_silu(proj, width, inner, channels, a.taps, a.conv_w, a.conv_b,
+                                     a.vector_dtype, a.state, a.slot_floats, step.state_slots,
+                                     step.token_seq, step.cu_q, xbc, m, step.num_seqs, l.stream()),
+               "causal_conv");
+    check_core(t.mk_ssm_scan(xbc, channels, proj, width, 0, inner + channels, a.dt_bias, a.a_log,
+                             a.d_skip, a.vector_dtype, a.state + a.carried_floats(), a.slot_floats,
+                             step.state_slots, step.cu_q, a.heads, a.vdim, a.state_size, a.groups,
+                             y, m, step.num_seqs, l.stream()), "ssm_scan");
+    check_core(t.mk_group_rmsnorm(y, normed, l.dtype(), a.norm, a.vector_dtype, a.eps, m, inner,
+                                  a.norm_groups, l.stream()), "group_rmsnorm");
+  }
+  project_into_stream(l, normed, m, a.w_out, hidden, inner, nullptr, kF32, h, pending,
+                      pending_count);
+}
+
+void normed_sum(Launch& l, float* h, const float* ya, const float* pa, int na, const void* wa,
+                const float* yb, const float* pb, int nb, const void* wb, int weight_dtype,
+                float eps, float mult, int tokens, int hidden) {
+  if (l.dry() || tokens == 0) return;
+  check_core(need_core().mk_normed_sum(h, ya, pa, na, wa, yb, pb, nb, wb, weight_dtype, eps, mult,
+                                       (long long)tokens * hidden, tokens, hidden, l.stream()),
+             "normed_sum");
+}
+
+void stream_mix(Launch& l, float* h, const float* kept, int m, int hidden, const void* w) {
+  void* both = l.alloc((size_t)m * 2 * hidden * l.elem());
+  if (l.dry() || m == 0) return;
+  check_core(need_core().mk_concat_cast(h, kept, both, l.dtype(), m, hidden, l.stream()),
+             "concat_cast");
+  linear(l, both, m, w, hidden, 2 * hidden, nullptr, kF32, h, kF32, false);
+}
+
+void copy_stream(Launch& l, float* dst, const float* src, long long n) {
+  if (l.dry() || n == 0) return;
+  check_core(need_core().mk_copy_f32(dst, src, n, l.stream()), "copy");
 }
 
 void* linear_per_head(Launch& l, const void* x, int m, int heads, int lda, int x_head,
@@ -498,7 +583,7 @@ void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scal
       check_core(need_core().mk_attention_generic_kv(
                      q.q, q.stride, out, a.heads * dv, a.k_cache, a.v_cache, l.dtype(), s.positions,
                      s.token_seq, s.table, s.table_stride, a.page_size, a.heads, 1, dk, dv, scale,
-                     0, 0.f, nullptr, m, l.stream()), "latent_attention");
+                     0, 0.f, nullptr, nullptr, m, l.stream()), "latent_attention");
     }
     return out;
   }

@@ -32,7 +32,7 @@ void embed(Launch& l, const int* ids, const void* table, int table_dtype, float*
 // adding `pending_count` partial sums [p, tokens, hidden] into h.
 void* rmsnorm(Launch& l, float* h, int tokens, int hidden, const float* pending, int pending_count,
               const void* weight, int weight_dtype, float eps, const int* rows, int out_rows,
-              void* out = nullptr);
+              void* out = nullptr, bool round_once = false);
 
 // The residual stream of a step of few tokens in fixed point (op_abi.h): its start, the norm
 // of rows of it, and a norm left for the projection behind it to fold in.
@@ -138,6 +138,27 @@ struct QkvForce {
 Queries qkv_project(Launch& l, const void* x, int m, int k, const QkvArgs& a, const StepArrays& s,
                     QkvForce force = {}, const NormFold* fold = nullptr);
 
+// What some makes of attention do to q and k between projection and cache, beyond a rotation:
+// RMS norms over the whole q and the whole k projection (weights q_norm [n_q d], k_norm
+// [n_kv d]), a query temperature 1 + coef * ln(floor((p + 1) / every) + 1), values that are
+// the keys as projected (no v rows in w), values of another width than the keys.
+struct QkPrep {
+  const void *q_norm = nullptr, *k_norm = nullptr;
+  int norm_dtype = 0;
+  float eps = 0.f;
+  float temp_coef = 0.f;
+  int temp_every = 0;
+  int values_are_keys = 0;
+  int value_dim = 0;            // 0: as wide as the keys
+  bool active() const {
+    return q_norm != nullptr || temp_every > 0 || values_are_keys != 0 || value_dim > 0;
+  }
+};
+// qkv_project for such an attention: the projection in float32, then one kernel for all of
+// the above, the rotation and the cache write.
+Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, const QkPrep& prep,
+                     const StepArrays& s);
+
 // Rotation and cache write of an already projected qkv [m, row_stride] (q rotated in place).
 void rope_kv_write(Launch& l, void* qkv, int row_stride, int m, const QkvArgs& a,
                    const StepArrays& s);
@@ -158,7 +179,11 @@ struct AttendArgs {
   // runs whatever the dtype.
   float score_cap = 0.f;
   const float* distance_slopes = nullptr;
-  bool plain_scores() const { return score_cap <= 0.f && distance_slopes == nullptr; }
+  // exp(sinks[head]) once more in the softmax's denominator (float32 [n_q])
+  const float* sinks = nullptr;
+  bool plain_scores() const {
+    return score_cap <= 0.f && distance_slopes == nullptr && sinks == nullptr;
+  }
 };
 
 struct AttendForce {
@@ -190,6 +215,44 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
 // `fold` as for qkv_project.
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
             int tile_config = -2, const NormFold* fold = nullptr, const GateAct& act = {});
+
+// h += act(x Wu^T) Wd^T for an activation of one operand (MK_UNARY_*), or partial sums left as
+// project_into_stream leaves them.
+void unary_mlp(Launch& l, const void* x, int m, int hidden, const void* w_up, const void* w_down,
+               int inter, int act, float* h, const float*& pending, int& pending_count);
+
+// A state-space mixer: in-projection [z | x | B | C | dt] in float32, the short convolution
+// over x, B, C with its carried inputs, the recurrence from the state earlier steps left, the
+// gate, the norm in groups, the output projection into h.  `state` holds, per slot of
+// `slot_floats` floats, the carried inputs followed by the recurrent state.
+struct StateSpaceArgs {
+  const void* w_in = nullptr;      // [2 inner + 2 groups N + heads, hidden]
+  const void *conv_w = nullptr, *conv_b = nullptr;   // [channels, taps], [channels]
+  const void *dt_bias = nullptr, *a_log = nullptr, *d_skip = nullptr;   // [heads]
+  const void* norm = nullptr;      // [inner]
+  int vector_dtype = 0;
+  const void* w_out = nullptr;     // [hidden, inner]
+  int heads = 0, vdim = 0, state_size = 0, groups = 0, taps = 0, norm_groups = 1;
+  float eps = 0.f;
+  float* state = nullptr;
+  long long slot_floats = 0;
+  int inner() const { return heads * vdim; }
+  int channels() const { return heads * vdim + 2 * groups * state_size; }
+  int in_width() const { return 2 * heads * vdim + 2 * groups * state_size + heads; }
+  long long carried_floats() const { return (long long)(taps - 1) * channels(); }
+};
+void state_space(Launch& l, const void* x, int m, int hidden, const StateSpaceArgs& a,
+                 const mk_step_view& step, float* h, const float*& pending, int& pending_count);
+
+// h += mult * (rmsnorm(a) wa + rmsnorm(b) wb), a = ya + its partial sums (see mk_normed_sum).
+void normed_sum(Launch& l, float* h, const float* ya, const float* pa, int na, const void* wa,
+                const float* yb, const float* pb, int nb, const void* wb, int weight_dtype,
+                float eps, float mult, int tokens, int hidden);
+
+// h <- [h | kept] W^T: the stream re-entered through a projection of itself beside a stream
+// kept from earlier in the step.
+void stream_mix(Launch& l, float* h, const float* kept, int m, int hidden, const void* w);
+void copy_stream(Launch& l, float* dst, const float* src, long long n);
 
 // y[t, head, :] = W[head] x[t, head, :] for every head: x rows `lda` apart with head `head`
 // at x + head * x_head, W [heads, n, k], y rows `ldo` apart with the head at out + head * o_head

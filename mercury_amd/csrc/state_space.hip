@@ -1,0 +1,310 @@
+// A state-space mixer (Mamba-2 make) in float32 arithmetic: the short causal convolution
+// with its carried inputs, the recurrence over a step's tokens from the state earlier steps
+// left, and the gated norm in groups behind it.
+//
+//   S_t = exp(-exp(A_log_h) dt_t) S_(t-1) + dt_t B_t x_t^T      (S is N x P per head)
+//   y_t = S_t^T C_t + D_h x_t,   dt_t = softplus(raw_t + dt_bias_h)
+//
+// A step runs the tokens it brings, in order, sequence by sequence; nothing distinguishes a
+// prompt portion from a decoded token, and the order of every sum depends on the sizes
+// alone, so a position's result does not depend on how its sequence was cut.
+//
+// The recurrence: a workgroup of four wavefronts owns 32 columns p of one head of one
+// sequence; a wavefront 8 columns x 8 slices of n, a lane a column and N/8 (padded to a
+// multiple of 4) entries of n, so that the sum over n is in-lane but for three exchanges.
+// B_t, C_t, x_t, dt_t and the decay of 16 tokens at a time are staged in LDS.  The state lies
+// in memory as the lanes hold it ([head][block of 8 columns][entry][lane]), so reading and
+// writing it is contiguous: a decoded token is one read and one write of the state.
+#include "common.h"
+#include "mercury_kernels.h"
+
+#define SS_TOKENS 16      // tokens staged at a time
+#define SS_COLS 32        // columns of a workgroup
+#define SS_MAX_NI 32      // entries of n a lane holds at most: N <= 256
+
+namespace {
+
+template <typename TW>
+__device__ __forceinline__ float weight_at(const void* w, int i) {
+  return Elem<TW>::load((const TW*)w + i);
+}
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.f + expf(-v)); }
+
+// out[t, c] = silu(bias[c] + sum_j w[c, j] u(t - (taps-1) + j)[c]) over the sequence's own
+// inputs u, those before this step's first token coming from `carried`
+// [slot, taps - 1, channels] (oldest first; zeros in a fresh slot).
+template <typename TW>
+__global__ void causal_conv_kernel(const float* __restrict__ proj, int row_stride, int col0,
+                                   int channels, int taps, const void* __restrict__ w,
+                                   const void* __restrict__ bias,
+                                   const float* __restrict__ carried, size_t slot_stride,
+                                   const int* __restrict__ slots,
+                                   const int* __restrict__ token_seq,
+                                   const int* __restrict__ cu_q, float* __restrict__ out) {
+  const int t = blockIdx.x;
+  const int seq = token_seq[t];
+  const int local = t - cu_q[seq];
+  const float* mine = carried + (size_t)slots[seq] * slot_stride;
+  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    float acc = weight_at<TW>(bias, c);
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;            // how many tokens before t
+      float u;
+      if (back <= local) {
+        u = proj[(size_t)(t - back) * row_stride + col0 + c];
+      } else {
+        // carried[k]: k = taps - 1 - (back - local)
+        u = mine[(size_t)(taps - 1 - (back - local)) * channels + c];
+      }
+      acc = fmaf(weight_at<TW>(w, c * taps + j), u, acc);
+    }
+    out[(size_t)t * channels + c] = silu_f(acc);
+  }
+}
+
+// After the convolution: the last taps - 1 inputs of every sequence become its carried ones.
+__global__ void conv_carry_kernel(const float* __restrict__ proj, int row_stride, int col0,
+                                  int channels, int taps, float* __restrict__ carried,
+                                  size_t slot_stride, const int* __restrict__ slots,
+                                  const int* __restrict__ cu_q) {
+  const int seq = blockIdx.x;
+  const int first = cu_q[seq], count = cu_q[seq + 1] - first;
+  float* mine = carried + (size_t)slots[seq] * slot_stride;
+  const int keep = taps - 1;
+  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    // ascending k: entry k takes what entry k + count held, or this step's input
+    for (int k = 0; k < keep; ++k) {
+      const int at = count - keep + k;   // index among this step's tokens
+      mine[(size_t)k * channels + c] =
+          at >= 0 ? proj[(size_t)(first + at) * row_stride + col0 + c]
+                  : mine[(size_t)(k + count) * channels + c];
+    }
+  }
+}
+
+// lane -> (column within the wavefront's 8, slice of n); entry i of a lane is
+// n = (i / 4) * 32 + slice * 4 + i % 4, so that four entries are one 16-byte LDS read and the
+// eight slices read 128 contiguous bytes.
+template <int NI, typename TW>
+__global__ __launch_bounds__(256) void ssm_scan_kernel(
+    const float* __restrict__ xbc, int xbc_stride, const float* __restrict__ proj,
+    int proj_stride, int z_col, int dt_col, const void* __restrict__ dt_bias,
+    const void* __restrict__ a_log, const void* __restrict__ d_skip, float* __restrict__ state,
+    size_t slot_stride, const int* __restrict__ slots, const int* __restrict__ cu_q, int heads,
+    int P, int N, int groups, float* __restrict__ y_out) {
+  constexpr int NPAD = NI * 8;
+  __shared__ __attribute__((aligned(16))) float sB[SS_TOKENS][NPAD];
+  __shared__ __attribute__((aligned(16))) float sC[SS_TOKENS][NPAD];
+  __shared__ float sX[SS_TOKENS][SS_COLS];
+  __shared__ float sZ[SS_TOKENS][SS_COLS];
+  __shared__ float sDt[SS_TOKENS], sDecay[SS_TOKENS];
+
+  const int seq = blockIdx.z, head = blockIdx.y, pblock = blockIdx.x;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int slice = lane >> 3, col_in_wave = lane & 7;
+  const int col = pblock * SS_COLS + wave * 8 + col_in_wave;   // column p of the head
+  const int group = head / (heads / groups);
+  const int inner = heads * P;
+  const int first = cu_q[seq], count = cu_q[seq + 1] - first;
+  const int blocks8 = (P + SS_COLS - 1) / SS_COLS * (SS_COLS / 8);   // whole workgroups
+
+  float* mine = state + (size_t)slots[seq] * slot_stride +
+                ((size_t)head * blocks8 + (size_t)pblock * 4 + wave) * NI * 64;
+  const bool live = pblock * SS_COLS + wave * 8 < P;    // the wavefront has columns at all
+  float S[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) S[i] = live ? mine[i * 64 + lane] : 0.f;
+
+  const float rate = expf(weight_at<TW>(a_log, head));
+  const float bias = weight_at<TW>(dt_bias, head);
+  const float skip = weight_at<TW>(d_skip, head);
+
+  for (int t0 = 0; t0 < count; t0 += SS_TOKENS) {
+    const int n_tok = min(SS_TOKENS, count - t0);
+    __syncthreads();
+    for (int idx = tid; idx < n_tok * NPAD; idx += 256) {
+      const int tt = idx / NPAD, n = idx - tt * NPAD;
+      const float* row = xbc + (size_t)(first + t0 + tt) * xbc_stride + inner;
+      sB[tt][n] = n < N ? row[group * N + n] : 0.f;
+      sC[tt][n] = n < N ? row[groups * N + group * N + n] : 0.f;
+    }
+    for (int idx = tid; idx < n_tok * SS_COLS; idx += 256) {
+      const int tt = idx / SS_COLS, c = idx - tt * SS_COLS;
+      const int p = pblock * SS_COLS + c;
+      const size_t tok = first + t0 + tt;
+      sX[tt][c] = p < P ? xbc[tok * xbc_stride + head * P + p] : 0.f;
+      sZ[tt][c] = p < P ? proj[tok * proj_stride + z_col + head * P + p] : 0.f;
+    }
+    if (tid < n_tok) {
+      const float raw = proj[(size_t)(first + t0 + tid) * proj_stride + dt_col + head] + bias;
+      // softplus without a clamp: log(1 + e^raw), written so that a large raw does not overflow
+      const float dt = raw > 0.f ? raw + log1pf(expf(-raw)) : log1pf(expf(raw));
+      sDt[tid] = dt;
+      sDecay[tid] = expf(-rate * dt);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < n_tok; ++tt) {
+      const float x = sX[tt][wave * 8 + col_in_wave];
+      const float dtx = sDt[tt] * x, decay = sDecay[tt];
+      float y = 0.f;
+#pragma unroll
+      for (int i4 = 0; i4 < NI / 4; ++i4) {
+        const float4 b = *(const float4*)&sB[tt][i4 * 32 + slice * 4];
+        const float4 c = *(const float4*)&sC[tt][i4 * 32 + slice * 4];
+        float* s = &S[i4 * 4];
+        s[0] = fmaf(decay, s[0], dtx * b.x);
+        s[1] = fmaf(decay, s[1], dtx * b.y);
+        s[2] = fmaf(decay, s[2], dtx * b.z);
+        s[3] = fmaf(decay, s[3], dtx * b.w);
+        y = fmaf(s[0], c.x, y);
+        y = fmaf(s[1], c.y, y);
+        y = fmaf(s[2], c.z, y);
+        y = fmaf(s[3], c.w, y);
+      }
+      y += __shfl_xor(y, 8, MK_WAVE);
+      y += __shfl_xor(y, 16, MK_WAVE);
+      y += __shfl_xor(y, 32, MK_WAVE);
+      if (slice == 0 && col < P) {
+        const float z = sZ[tt][wave * 8 + col_in_wave];
+        y_out[(size_t)(first + t0 + tt) * inner + head * P + col] = (y + skip * x) * silu_f(z);
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) mine[i * 64 + lane] = S[i];
+  }
+}
+
+// One workgroup per (token, part): out = y / rms(part of y) * weight.
+template <typename T, typename TW>
+__global__ void group_norm_kernel(const float* __restrict__ y, T* __restrict__ out,
+                                  const void* __restrict__ weight, float eps, int width,
+                                  int parts) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, part = blockIdx.y;
+  const int size = width / parts;
+  const float* src = y + (size_t)t * width + (size_t)part * size;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < size; i += blockDim.x) sq += src[i] * src[i];
+  const float r = rsqrtf(block_sum(sq, scratch) / (float)size + eps);
+  for (int i = threadIdx.x; i < size; i += blockDim.x) {
+    Elem<T>::store(out + (size_t)t * width + (size_t)part * size + i,
+                   src[i] * r * weight_at<TW>(weight, part * size + i));
+  }
+}
+
+int entries_for(int N) {
+  int ni = (N + 7) / 8;
+  int padded = 4;
+  while (padded < ni) padded *= 2;
+  return padded;
+}
+
+}  // namespace
+
+// Floats of recurrent state one head occupies, as the kernel lays it out.
+extern "C" long long mk_ssm_state_floats(int heads, int P, int N) {
+  if (heads <= 0 || P <= 0 || N <= 0 || N > SS_MAX_NI * 8) return -1;
+  // whole workgroups of 32 columns, so that every wavefront's block exists
+  const long long blocks8 = (long long)((P + SS_COLS - 1) / SS_COLS) * (SS_COLS / 8);
+  return (long long)heads * blocks8 * entries_for(N) * 64;
+}
+
+extern "C" int mk_causal_conv_silu(const float* proj, int row_stride, int col0, int channels,
+                                   int taps, const void* w, const void* bias, int weight_dtype,
+                                   float* carried, long long slot_stride, const int* slots,
+                                   const int* token_seq, const int* cu_q, float* out, int tokens,
+                                   int num_seqs, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && num_seqs >= 0 && channels > 0 && taps >= 1, "causal_conv: bad sizes");
+  MK_REQUIRE(col0 >= 0 && row_stride >= col0 + channels, "causal_conv: columns outside the row");
+  MK_REQUIRE(slot_stride >= (long long)(taps - 1) * channels,
+             "causal_conv: a slot of %lld floats does not hold %d x %d carried inputs",
+             slot_stride, taps - 1, channels);
+  MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "causal_conv: weight dtype %d",
+             weight_dtype);
+  if (tokens == 0) return 0;
+  if (weight_dtype == MK_F32)
+    causal_conv_kernel<float><<<tokens, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
+                                                           w, bias, carried, (size_t)slot_stride,
+                                                           slots, token_seq, cu_q, out);
+  else
+    causal_conv_kernel<bf16_t><<<tokens, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
+                                                            w, bias, carried, (size_t)slot_stride,
+                                                            slots, token_seq, cu_q, out);
+  MK_LAUNCH_CHECK("causal_conv");
+  if (taps > 1) {
+    conv_carry_kernel<<<num_seqs, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
+                                                    carried, (size_t)slot_stride, slots, cu_q);
+    MK_LAUNCH_CHECK("conv_carry");
+  }
+  return 0;
+}
+
+extern "C" int mk_ssm_scan(const float* xbc, int xbc_stride, const float* proj, int proj_stride,
+                           int z_col, int dt_col, const void* dt_bias, const void* a_log,
+                           const void* d_skip, int weight_dtype, float* state,
+                           long long slot_stride, const int* slots, const int* cu_q, int heads,
+                           int P, int N, int groups, float* y_out, int tokens, int num_seqs,
+                           hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && num_seqs >= 0 && heads > 0 && P > 0 && N > 0 && groups > 0,
+             "ssm_scan: bad sizes");
+  MK_REQUIRE(heads % groups == 0, "ssm_scan: %d heads are not a multiple of %d groups", heads, groups);
+  MK_REQUIRE(N <= SS_MAX_NI * 8, "ssm_scan: state size %d exceeds %d", N, SS_MAX_NI * 8);
+  MK_REQUIRE(slot_stride >= mk_ssm_state_floats(heads, P, N),
+             "ssm_scan: a slot of %lld floats does not hold the state", slot_stride);
+  MK_REQUIRE(xbc_stride >= heads * P + 2 * groups * N, "ssm_scan: x, B, C outside the row");
+  MK_REQUIRE(z_col >= 0 && dt_col >= 0 && proj_stride >= z_col + heads * P &&
+                 proj_stride >= dt_col + heads, "ssm_scan: gate or step sizes outside the row");
+  MK_REQUIRE(heads <= 65535 && num_seqs <= 65535, "ssm_scan: too many heads or sequences");
+  MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "ssm_scan: weight dtype %d",
+             weight_dtype);
+  if (tokens == 0 || num_seqs == 0) return 0;
+  const dim3 grid((P + SS_COLS - 1) / SS_COLS, heads, num_seqs);
+  const int ni = entries_for(N);
+#define SS_LAUNCH(NI)                                                                          \
+  do {                                                                                         \
+    if (weight_dtype == MK_F32)                                                                \
+      ssm_scan_kernel<NI, float><<<grid, 256, 0, stream>>>(                                    \
+          xbc, xbc_stride, proj, proj_stride, z_col, dt_col, dt_bias, a_log, d_skip, state,    \
+          (size_t)slot_stride, slots, cu_q, heads, P, N, groups, y_out);                       \
+    else                                                                                       \
+      ssm_scan_kernel<NI, bf16_t><<<grid, 256, 0, stream>>>(                                   \
+          xbc, xbc_stride, proj, proj_stride, z_col, dt_col, dt_bias, a_log, d_skip, state,    \
+          (size_t)slot_stride, slots, cu_q, heads, P, N, groups, y_out);                       \
+  } while (0)
+  if (ni == 4) SS_LAUNCH(4);
+  else if (ni == 8) SS_LAUNCH(8);
+  else if (ni == 16) SS_LAUNCH(16);
+  else SS_LAUNCH(32);
+#undef SS_LAUNCH
+  MK_LAUNCH_CHECK("ssm_scan");
+  return 0;
+}
+
+extern "C" int mk_group_rmsnorm(const float* y, void* out, int dtype, const void* weight,
+                                int weight_dtype, float eps, int tokens, int width, int parts,
+                                hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && width > 0 && parts > 0 && width % parts == 0,
+             "group_rmsnorm: %d columns in %d parts", width, parts);
+  MK_REQUIRE(parts <= 65535, "group_rmsnorm: too many parts");
+  MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "group_rmsnorm: weight dtype %d",
+             weight_dtype);
+  if (tokens == 0) return 0;
+  const dim3 grid(tokens, parts);
+  const int size = width / parts;
+  const int threads = size >= 1024 ? 256 : (size >= 256 ? 128 : 64);
+#define GN_LAUNCH(T, TW)                                                            \
+  group_norm_kernel<T, TW><<<grid, threads, 0, stream>>>(y, (T*)out, weight, eps, width, parts)
+  if (dtype == MK_F32) {
+    if (weight_dtype == MK_F32) GN_LAUNCH(float, float); else GN_LAUNCH(float, bf16_t);
+  } else if (dtype == MK_BF16) {
+    if (weight_dtype == MK_F32) GN_LAUNCH(bf16_t, float); else GN_LAUNCH(bf16_t, bf16_t);
+  } else {
+    MK_REQUIRE(false, "group_rmsnorm: unknown dtype %d", dtype);
+  }
+#undef GN_LAUNCH
+  MK_LAUNCH_CHECK("group_rmsnorm");
+  return 0;
+}

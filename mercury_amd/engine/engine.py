@@ -190,9 +190,9 @@ class Engine:
         groups = {slot: sizing.group_of(slot) for slot in model.cache_slots}
         model.prepare(cfg.max_model_len, device)
         caches = sizing_caches(model, groups, cfg.block_size, cfg.torch_dtype, device)
-        states = {i: torch.empty((0, *layer.mixer.state_spec().shape),
-                                 dtype=layer.mixer.state_spec().dtype, device=device)
-                  for i, layer in enumerate(model.layers) if layer.mixer.state_spec() is not None}
+        specs = {n: model.layers[call.layer].mixer.state_spec() for n, call in enumerate(model.calls)}
+        states = {n: torch.empty((0, *spec.shape), dtype=spec.dtype, device=device)
+                  for n, spec in specs.items() if spec is not None}
         program = model.compile(caches, states)
         needs = ModelRunner.step_needs(program, max(1, sizing.num_groups), cfg.block_size,
                                        cfg.max_model_len, min(cfg.prefill_budget, cfg.max_model_len),

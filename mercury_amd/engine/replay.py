@@ -11,7 +11,9 @@ pass, cache or loader.
 ``--max-tokens`` is the most tokens that live requests hold at any time, each request's count
 rounded up to a multiple of 64 (of the page size, if that is larger); the cache pool is made
 for exactly this many, so that pages are used again.  ``--block-size`` is the page size of the
-cache (a power of two, default 16), ``--max-live`` the most requests live at a time.
+cache (a power of two, default 16), ``--max-live`` the most requests live at a time (default 4;
+a model whose mixers carry per-request state has that many state slots, used again as
+requests end).
 
 Input (standard input, one JSON object per line):
 
@@ -30,7 +32,7 @@ import sys
 from pathlib import Path
 
 DEFAULT_PAGE_SIZE = 16     # the engine's default block_size
-DEFAULT_MAX_LIVE = 8
+DEFAULT_MAX_LIVE = 4       # also the number of state slots of a model whose mixers carry state
 ROUNDING = 64              # a live request counts as its length rounded up to this many tokens
 
 

@@ -90,10 +90,15 @@ class DecodeGraph:
         stream = torch.cuda.current_stream(runner.device)
         runner.packer.upload(packed, buffers.ints.data_ptr(), stream.cuda_stream)
         # Once outside the capture (loads libraries, warms the kernels), then captured.
+        # Writing keys and values twice is harmless; advancing per-request state twice is not,
+        # so the state is put back as it was before the graph runs the step for good.
         side = torch.cuda.Stream(device=runner.device)
         side.wait_stream(stream)
         with torch.cuda.stream(side):
+            before = {n: state.clone() for n, state in runner.states.items()}
             runner.launch(packed, buffers)
+            for n, state in runner.states.items():
+                state.copy_(before[n])
         stream.wait_stream(side)
         torch.cuda.synchronize(runner.device)
         self.graph = torch.cuda.CUDAGraph()
@@ -166,12 +171,13 @@ class ModelRunner:
             k, v = self.kv[call.cache]
             self.caches[n] = LayerCache(k, v, manager.group_of(call.cache), self.page_size,
                                         call.writes)
-        # Per-request state of fixed size, one tensor per layer that declares it.
+        # Per-request state of fixed size, one tensor per execution-list entry whose mixer
+        # declares it (a layer that runs twice carries two states).
         self.states = {}
-        for i, layer in enumerate(model.layers):
-            spec = layer.mixer.state_spec()
+        for n, call in enumerate(model.calls):
+            spec = model.layers[call.layer].mixer.state_spec()
             if spec is not None:
-                self.states[i] = torch.zeros((manager.state_slots.num_slots, *spec.shape),
+                self.states[n] = torch.zeros((manager.state_slots.num_slots, *spec.shape),
                                              dtype=spec.dtype, device=device)
         # The model as a program of the host core; parts that do not hand their work over
         # are steps this runner runs in between (model.caller_steps).

@@ -33,6 +33,8 @@ LIBRARIES = {
         "attention_generic.hip",
         "latent.hip",
         "experts.hip",
+        "mixers.hip",
+        "state_space.hip",
         "sampling.hip",
         "random_fill.hip",
     ],

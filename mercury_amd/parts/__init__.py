@@ -6,12 +6,15 @@ from .base import (CacheSpec, FeedForward, LayerCache, Mixer, Norm, Part, Positi
 from .block import ParallelBlock, PreNormBlock
 from .embedding import OutputHead, TokenEmbedding
 from .experts import RoutedExperts
-from .feedforward import GatedMLP
+from .feedforward import GatedMLP, UnaryMLP
 from .latent_attention import LatentAttention
 from .lowering import OneOp
+from .mixer_sum import NormedMixerSum
 from .model import CallerStep, DecoderModel, LayerCall, Registers
 from .norm import RMSNorm
 from .position import NoPosition, RotaryPosition
+from .state_space import StateSpaceMixer
+from .stream_mix import StreamMix
 from .registry import (build_part, known, register_block, register_ffn, register_mixer,
                        register_norm, register_position)
 
@@ -19,6 +22,9 @@ register_mixer("attention")(Attention)
 register_mixer("latent_attention")(LatentAttention)
 register_ffn("gated_mlp")(GatedMLP)
 register_ffn("routed_experts")(RoutedExperts)
+register_ffn("unary_mlp")(UnaryMLP)
+register_mixer("state_space")(StateSpaceMixer)
+register_mixer("normed_sum")(NormedMixerSum)
 register_norm("rmsnorm")(RMSNorm)
 register_position("rotary")(RotaryPosition)
 register_position("none")(NoPosition)
@@ -29,7 +35,7 @@ __all__ = [
     "Attention", "CacheSpec", "CallerStep", "DecoderModel", "FeedForward", "GatedMLP",
     "LatentAttention", "LayerCache", "LayerCall", "Mixer", "NoPosition", "Norm", "OneOp", "OutputHead", "Part",
     "ParallelBlock", "PositionDescriptor", "PositionEncoding", "PreNormBlock", "Registers",
-    "RoutedExperts",
+    "RoutedExperts", "NormedMixerSum", "StateSpaceMixer", "StreamMix", "UnaryMLP",
     "RMSNorm", "RotaryPosition", "StateSpec", "TensorSpec", "TokenEmbedding", "build_part", "known",
     "register_block", "register_ffn", "register_mixer", "register_norm", "register_position",
 ]

@@ -11,7 +11,8 @@ from .lowering import OneOp
 
 # Leaf names of the stored tensors, under the prefix the builder gives; an architecture whose
 # checkpoints call them otherwise passes its own map.
-DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj"}
+DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj",
+                 "q_norm": "q_norm", "k_norm": "k_norm", "sink": "sink"}
 
 
 class Attention(Mixer):
@@ -26,6 +27,18 @@ class Attention(Mixer):
     `score_cap` bounds the scaled score to cap * tanh(score / cap); a position encoding may
     bring a penalty on the distance in the score (`PositionDescriptor.distance_slopes`).  The
     reference has neither; with either the float32-arithmetic attention kernel runs.
+
+    Further makes of the same mixer, each a parameter:
+    `values="keys"`: there is no v projection; the values are the keys as projected (with their
+    bias), before any norm or rotation.  `value_dim`: values of another width than the keys.
+    `qk_norm` ("whole"): an RMS norm over the whole q projection and one over the whole k
+    projection (all heads at once; plain weights ``<q_norm>.weight`` [n_q d] and
+    ``<k_norm>.weight`` [n_kv d], eps `norm_eps`), before the rotation.
+    `q_temp=(coef, every)`: the query at position p is multiplied by
+    1 + coef * ln(floor((p + 1) / every) + 1), after its norm.
+    `sinks`: a stored number per query head (``<sink>.weight`` [n_q]) whose exponential stands
+    once more in the softmax's denominator, unscaled, with no key or value behind it.
+    `k_bias` / `v_bias` (default: as `qkv_bias`) say which of the projections have a bias.
     """
 
     graph_safe = True   # forward launches kernels only: a decode step may be captured in a graph
@@ -33,7 +46,10 @@ class Attention(Mixer):
     def __init__(self, hidden: int, n_q: int, n_kv: int, head_dim: int,
                  position: PositionEncoding, qkv_bias: bool = True, o_bias: bool = False,
                  scale: float | None = None, window: int | None = None,
-                 names: dict | None = None, score_cap: float | None = None):
+                 names: dict | None = None, score_cap: float | None = None,
+                 values: str = "projected", value_dim: int | None = None,
+                 qk_norm: str | None = None, norm_eps: float = 1e-6,
+                 q_temp: tuple | None = None, sinks: bool = False):
         if n_q % n_kv:
             raise ValueError(f"{n_q} query heads are not a multiple of {n_kv} key/value heads")
         self.hidden, self.n_q, self.n_kv, self.head_dim = int(hidden), int(n_q), int(n_kv), int(head_dim)
@@ -42,44 +58,80 @@ class Attention(Mixer):
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
         self.window = int(window) if window else None
         self.score_cap = float(score_cap) if score_cap else 0.0
+        if values not in ("projected", "keys"):
+            raise ValueError(f"values {values!r}: 'projected' or 'keys'")
+        self.values_are_keys = values == "keys"
+        self.value_dim = int(value_dim) if value_dim else self.head_dim
+        if self.values_are_keys and self.value_dim != self.head_dim:
+            raise ValueError("values that are the keys are as wide as the keys")
+        if qk_norm not in (None, "whole"):
+            raise ValueError(f"qk_norm {qk_norm!r}: None or 'whole'")
+        self.qk_norm, self.norm_eps = qk_norm, float(norm_eps)
+        self.q_temp = (float(q_temp[0]), int(q_temp[1])) if q_temp else None
+        if self.q_temp and self.q_temp[1] <= 0:
+            raise ValueError("the query temperature's period must be positive")
+        self.sinks = bool(sinks)
         self.names = {**DEFAULT_NAMES, **(names or {})}
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+        self.w_q_norm = self.w_k_norm = self.sink = None
         self._alone: dict = {}
+
+    @property
+    def prepared(self) -> bool:
+        """Whether q and k get more than a rotation between projection and cache (the kernels
+        then take the projection in float32 and do all of it in one pass)."""
+        return bool(self.values_are_keys or self.qk_norm or self.q_temp
+                    or self.value_dim != self.head_dim)
 
     # ---- declarations
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(self.n_kv, self.head_dim, self.window)
+        value_dim = None if self.value_dim == self.head_dim else self.value_dim
+        return CacheSpec(self.n_kv, self.head_dim, self.window, value_dim)
+
+    def _projections(self) -> list:
+        """The stacked projections in order: (name key, rows)."""
+        out = [("q", self.n_q * self.head_dim), ("k", self.n_kv * self.head_dim)]
+        if not self.values_are_keys:
+            out.append(("v", self.n_kv * self.value_dim))
+        return out
 
     def param_specs(self) -> dict:
-        q, kv, h = self.n_q * self.head_dim, self.n_kv * self.head_dim, self.hidden
-        n = self.names
-        specs = {
-            f"{n['q']}.weight": TensorSpec((q, h)),
-            f"{n['k']}.weight": TensorSpec((kv, h)),
-            f"{n['v']}.weight": TensorSpec((kv, h)),
-            f"{n['o']}.weight": TensorSpec((h, q)),
-        }
-        if self.qkv_bias:
-            specs[f"{n['q']}.bias"] = TensorSpec((q,), role="vector")
-            specs[f"{n['k']}.bias"] = TensorSpec((kv,), role="vector")
-            specs[f"{n['v']}.bias"] = TensorSpec((kv,), role="vector")
+        h, n = self.hidden, self.names
+        specs = {}
+        for key, rows in self._projections():
+            specs[f"{n[key]}.weight"] = TensorSpec((rows, h))
+            if self.qkv_bias:
+                specs[f"{n[key]}.bias"] = TensorSpec((rows,), role="vector")
+        specs[f"{n['o']}.weight"] = TensorSpec((h, self.n_q * self.value_dim))
         if self.o_bias:
             specs[f"{n['o']}.bias"] = TensorSpec((h,), role="vector")
+        if self.qk_norm:
+            specs[f"{n['q_norm']}.weight"] = TensorSpec((self.n_q * self.head_dim,), role="vector",
+                                                        init="one_plus_normal")
+            specs[f"{n['k_norm']}.weight"] = TensorSpec((self.n_kv * self.head_dim,), role="vector",
+                                                        init="one_plus_normal")
+        if self.sinks:
+            specs[f"{n['sink']}.weight"] = TensorSpec((self.n_q,), role="vector")
         return specs
 
     def bind(self, params, dtype, device) -> None:
         n = self.names
         # One projection for q, k and v: rows [q heads | k heads | v heads].
-        self.w_qkv = torch.cat(
-            [params[f"{n['q']}.weight"], params[f"{n['k']}.weight"], params[f"{n['v']}.weight"]],
-            dim=0).contiguous()
+        keys = [key for key, _rows in self._projections()]
+        self.w_qkv = torch.cat([params[f"{n[key]}.weight"] for key in keys], dim=0).contiguous()
         if self.qkv_bias:
-            biases = [params[f"{n['q']}.bias"], params[f"{n['k']}.bias"], params[f"{n['v']}.bias"]]
+            biases = [params[f"{n[key]}.bias"] for key in keys]
             common = torch.float32 if any(b.dtype == torch.float32 for b in biases) else dtype
             self.b_qkv = torch.cat([b.to(common) for b in biases]).contiguous()
         self.w_o = params[f"{n['o']}.weight"]
         self.b_o = params.get(f"{n['o']}.bias")
+        if self.qk_norm:
+            # both in float32: one dtype code for the two
+            self.w_q_norm = params[f"{n['q_norm']}.weight"].float().contiguous()
+            self.w_k_norm = params[f"{n['k_norm']}.weight"].float().contiguous()
+        if self.sinks:
+            self.sink = params[f"{n['sink']}.weight"].float().contiguous()
         self._alone.clear()
 
     def prepare(self, max_positions: int, device) -> None:
@@ -87,7 +139,8 @@ class Attention(Mixer):
 
     def weight_bytes(self) -> int:
         total = 0
-        for t in (self.w_qkv, self.b_qkv, self.w_o, self.b_o):
+        for t in (self.w_qkv, self.b_qkv, self.w_o, self.b_o, self.w_q_norm, self.w_k_norm,
+                  self.sink):
             if t is not None:
                 total += t.numel() * t.element_size()
         return total
@@ -104,9 +157,6 @@ class Attention(Mixer):
         pos = self.position.describe()
         if pos is None:
             raise ValueError("an attention whose position encoding applies itself is not lowered")
-        spec = self.cache_spec()
-        if spec.v_dim != self.head_dim:
-            raise ValueError("the attention kernels keep values as wide as keys")
         if cache.k.dtype != self.w_qkv.dtype:
             raise ValueError("the kernels keep keys and values in the compute dtype")
         bias_code = lambda t: ops.dtype_code(t.dtype) if t is not None else ops.F32
@@ -125,7 +175,12 @@ class Attention(Mixer):
             interleaved=pos.interleaved, k_cache=cache.k.data_ptr(), v_cache=cache.v.data_ptr(),
             group=cache.group, page_size=cache.page_size, scale=self.scale,
             window=self.window or 0, writes=cache.writes, score_cap=self.score_cap,
-            distance_slopes=ptr(pos.distance_slopes)))
+            distance_slopes=ptr(pos.distance_slopes), sinks=ptr(self.sink),
+            q_norm=ptr(self.w_q_norm), k_norm=ptr(self.w_k_norm), norm_dtype=ops.F32,
+            norm_eps=self.norm_eps, temp_coef=self.q_temp[0] if self.q_temp else 0.0,
+            temp_every=self.q_temp[1] if self.q_temp else 0,
+            values_are_keys=self.values_are_keys,
+            value_dim=self.value_dim if self.prepared else 0))
 
     def forward(self, x, step, cache, state, accum):
         if self.position.describe() is not None:
@@ -137,6 +192,9 @@ class Attention(Mixer):
                                                  lambda program: self.lower(program, cache))
             _logits, _x, pending = alone.run(step, accum, x=x)
             return pending
+        if self.prepared or self.sinks:
+            raise ValueError("an attention with norms over q and k, a query temperature, sinks "
+                             "or values that are keys needs a position encoding the kernels apply")
         # The encoding applies itself: project, let it transform q and k where they lie, then
         # write keys and values to the cache as they are.
         n_q, n_kv, d = self.n_q, self.n_kv, self.head_dim

@@ -73,3 +73,54 @@ class GatedMLP(FeedForward):
             self._alone = OneOp(x.dtype, self.hidden, 0, self.lower)
         _logits, _x, pending = self._alone.run(step, accum, x=x)
         return pending
+
+
+UNARY_ACTIVATIONS = {"relu2": 0}     # the kernels' codes
+UNARY_NAMES = {"up": "up_proj", "down": "down_proj"}
+
+
+class UnaryMLP(FeedForward):
+    """down(act(up(x))) without biases, for an activation of one operand.  `activation`:
+
+    ``"relu2"``: the square of relu.
+
+    `names` maps up, down to the stored tensors' leaf names (default ``up_proj``,
+    ``down_proj``)."""
+
+    graph_safe = True
+    lowerable = True
+
+    def __init__(self, hidden: int, intermediate: int, activation: str = "relu2",
+                 names: dict | None = None):
+        if activation not in UNARY_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not implemented; known: "
+                             f"{sorted(UNARY_ACTIVATIONS)}")
+        self.hidden, self.intermediate = int(hidden), int(intermediate)
+        self.activation = activation
+        self.names = {**UNARY_NAMES, **(names or {})}
+        self.w_up = self.w_down = None
+        self._alone = None
+
+    def param_specs(self) -> dict:
+        i, h, n = self.intermediate, self.hidden, self.names
+        return {f"{n['up']}.weight": TensorSpec((i, h)), f"{n['down']}.weight": TensorSpec((h, i))}
+
+    def bind(self, params, dtype, device) -> None:
+        n = self.names
+        self.w_up = params[f"{n['up']}.weight"]
+        self.w_down = params[f"{n['down']}.weight"]
+        self._alone = None
+
+    def weight_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.w_up, self.w_down))
+
+    def lower(self, program) -> None:
+        program.append("unary_mlp", core.unary_mlp_params(
+            self.w_up.data_ptr(), self.w_down.data_ptr(), self.intermediate,
+            act=UNARY_ACTIVATIONS[self.activation]))
+
+    def forward(self, x, step, accum):
+        if self._alone is None:
+            self._alone = OneOp(x.dtype, self.hidden, 0, self.lower)
+        _logits, _x, pending = self._alone.run(step, accum, x=x)
+        return pending

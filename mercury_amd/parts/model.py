@@ -23,11 +23,18 @@ class LayerCall:
     writes
         whether this call writes its tokens' keys and values into the slot; a call that only
         reads attends over what the writing call stored earlier in the same step.
+    mix
+        the model's `stream_mix` part runs right before this call (the stream re-enters
+        through a projection of itself beside the embedding output).
+
+    A mixer's per-request state belongs to the entry, not to the layer: a layer named twice
+    carries two states.
     """
 
     layer: int
     cache: int | None
     writes: bool = True
+    mix: bool = False
 
 
 @dataclass
@@ -68,7 +75,8 @@ class DecoderModel(Part):
                  norm_prefix: str = "model.norm.", head_name: str = "lm_head.weight",
                  max_positions: int = 0, eos_token_ids: tuple = (), config=None,
                  embedding: Part | None = None, head: Part | None = None,
-                 layer_ids: list | None = None, stored_name=None):
+                 layer_ids: list | None = None, stored_name=None,
+                 stream_mix: Part | None = None, mix_prefix: str = "stream_mix."):
         """`layer_ids`: the index each layer's tensors are stored under (default: its place in
         `layers`), for a model some of whose executed layers own no tensors.  `stored_name`:
         a function from a tensor's name as the parts compose it (prefixes + the part's leaf,
@@ -79,6 +87,7 @@ class DecoderModel(Part):
         if len(self.layer_ids) != len(self.layers):
             raise ValueError("one stored index per layer")
         self.stored_name = stored_name
+        self.stream_mix, self.mix_prefix = stream_mix, mix_prefix
         self.final_norm = final_norm
         self.tied_head = bool(tied_head)
         self.calls = list(calls) if calls is not None else [
@@ -103,6 +112,9 @@ class DecoderModel(Part):
 
     def _check_calls(self) -> None:
         writers = {}
+        if any(call.mix for call in self.calls) and self.stream_mix is None:
+            raise ValueError("an execution list entry re-enters the stream, but the model has "
+                             "no stream_mix part")
         for n, call in enumerate(self.calls):
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"execution list entry {n} names layer {call.layer}")
@@ -144,6 +156,9 @@ class DecoderModel(Part):
             prefix = self.layer_prefix.format(i)
             for name, spec in layer.param_specs().items():
                 specs[prefix + name] = spec
+        if self.stream_mix is not None:
+            for name, spec in self.stream_mix.param_specs().items():
+                specs[self.mix_prefix + name] = spec
         for name, spec in self.final_norm.param_specs().items():
             specs[self.norm_prefix + name] = spec
         for name, spec in self.head_part.param_specs().items():
@@ -165,6 +180,8 @@ class DecoderModel(Part):
         self.head = head_params["weight"]
         for i, layer in zip(self.layer_ids, self.layers):
             layer.bind(under(self.layer_prefix.format(i)), dtype, device)
+        if self.stream_mix is not None:
+            self.stream_mix.bind(under(self.mix_prefix), dtype, device)
         self.final_norm.bind(under(self.norm_prefix), dtype, device)
 
     def prepare(self, max_positions: int, device) -> None:
@@ -184,6 +201,8 @@ class DecoderModel(Part):
         """Bytes of weights a step reads once: every layer the execution list runs, the final
         norm and the head (the embedding is gathered, not streamed)."""
         total = sum(self.layers[c.layer].weight_bytes() for c in self.calls)
+        if self.stream_mix is not None:
+            total += self.stream_mix.weight_bytes() * sum(1 for c in self.calls if c.mix)
         total += self.final_norm.weight_bytes()
         total += self.head_part.weight_bytes()
         return total
@@ -191,7 +210,9 @@ class DecoderModel(Part):
     # ---- as a program of the host core
 
     def compile(self, caches: dict, states: dict):
-        """The step as a program: the embedding, every execution-list entry, the final norm
+        """`caches` and `states` are keyed by the execution-list index.
+
+        The step as a program: the embedding, every execution-list entry, the final norm
         over the wanted rows, the head.  A part that hands its work over appends its
         operations; any other becomes a step the caller runs (`caller_steps`, by index), on
         the same registers, between two stretches of the program."""
@@ -208,9 +229,13 @@ class DecoderModel(Part):
             self.embedding_part.lower(program)
         else:
             stays(lambda r: self.embedding_part.forward(r.step, out=r.h), "embedding")
+        if self.stream_mix is not None:
+            self.stream_mix.lower_keep(program)
         for n, call in enumerate(self.calls):
             layer = self.layers[call.layer]
-            cache, state = caches.get(n), states.get(call.layer)
+            cache, state = caches.get(n), states.get(n)
+            if call.mix:
+                self.stream_mix.lower(program)
             can = getattr(layer, "lowerable_with", None)
             if can is not None and can(state):
                 if state is None:
