@@ -212,8 +212,10 @@ int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int dtype, cons
                   int page_size, int n_q, int n_kv, int d, int dv, int values_are_keys,
                   int write_kv, int tokens, hipStream_t stream);
 
-// out[i] = act(x[i]) for an activation MK_UNARY_*.
-int mk_unary_act(const void* x, void* out, int dtype, long long n, int kind, hipStream_t stream);
+// out[i] = act(x[i]) for an activation MK_UNARY_*; x of in_dtype (float32, or the output's),
+// the result rounded once to `dtype`.
+int mk_unary_act(const void* x, int in_dtype, void* out, int dtype, long long n, int kind,
+                 hipStream_t stream);
 
 // h[t, :] += mult * (rmsnorm(a[t, :]) * wa + rmsnorm(b[t, :]) * wb), with a = ya + its `na`
 // partial sums pa[k * stride + .] (ya may be null) and b likewise (no b at all: yb null and

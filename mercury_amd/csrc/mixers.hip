@@ -99,12 +99,12 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   }
 }
 
-template <typename T>
-__global__ void unary_act_kernel(const T* __restrict__ x, T* __restrict__ out, long long n,
+template <typename TI, typename T>
+__global__ void unary_act_kernel(const TI* __restrict__ x, T* __restrict__ out, long long n,
                                  int kind) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const float v = Elem<T>::load(x + i);
+  const float v = Elem<TI>::load(x + i);
   float y = v;
   if (kind == MK_UNARY_RELU2) {
     const float r = fmaxf(v, 0.f);
@@ -204,19 +204,21 @@ extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int 
   return 0;
 }
 
-extern "C" int mk_unary_act(const void* x, void* out, int dtype, long long n, int kind,
-                            hipStream_t stream) {
+extern "C" int mk_unary_act(const void* x, int in_dtype, void* out, int dtype, long long n,
+                            int kind, hipStream_t stream) {
   MK_REQUIRE(n >= 0, "unary_act: negative count");
   MK_REQUIRE(kind == MK_UNARY_RELU2, "unary_act: unknown activation %d", kind);
   if (n == 0) return 0;
   const long long blocks = (n + 255) / 256;
   MK_REQUIRE(blocks < (1ll << 31), "unary_act: %lld elements are too many for one launch", n);
-  if (dtype == MK_F32)
-    unary_act_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)x, (float*)out, n, kind);
-  else if (dtype == MK_BF16)
-    unary_act_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, n, kind);
+  if (in_dtype == MK_F32 && dtype == MK_F32)
+    unary_act_kernel<float, float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)x, (float*)out, n, kind);
+  else if (in_dtype == MK_F32 && dtype == MK_BF16)
+    unary_act_kernel<float, bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const float*)x, (bf16_t*)out, n, kind);
+  else if (in_dtype == MK_BF16 && dtype == MK_BF16)
+    unary_act_kernel<bf16_t, bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, n, kind);
   else
-    MK_REQUIRE(false, "unary_act: unknown dtype %d", dtype);
+    MK_REQUIRE(false, "unary_act: dtypes %d -> %d", in_dtype, dtype);
   MK_LAUNCH_CHECK("unary_act");
   return 0;
 }

@@ -283,6 +283,8 @@ int run_keep_stream(const void*, mk_op_context* ctx) {
   return guarded(ctx, [&] {
     Launch l(ctx);
     if (!l.dry() && !ctx->kept) throw KernelError("keep_stream: the step has no room to keep a stream");
+    const long long n = (long long)ctx->step->num_tokens * ctx->hidden;
+    if (ctx->pending_count > 0) scaled_add(l, ctx->h, nullptr, ctx->pending, ctx->pending_count, nullptr, 0, n, 1.f);
     copy_stream(l, ctx->kept, ctx->h, (long long)ctx->step->num_tokens * ctx->hidden);
   });
 }
@@ -292,6 +294,9 @@ int run_stream_mix(const void* params, mk_op_context* ctx) {
     const StreamMixParams& p = *static_cast<const StreamMixParams*>(params);
     Launch l(ctx);
     if (!l.dry() && !ctx->kept) throw KernelError("stream_mix: no stream was kept in this step");
+    const long long n = (long long)ctx->step->num_tokens * ctx->hidden;
+    // what the projection before left as partial sums belongs to the stream first
+    if (ctx->pending_count > 0) scaled_add(l, ctx->h, nullptr, ctx->pending, ctx->pending_count, nullptr, 0, n, 1.f);
     stream_mix(l, ctx->h, ctx->kept, ctx->step->num_tokens, ctx->hidden, p.weight);
   });
 }
@@ -392,8 +397,8 @@ void register_builtin_ops() {
   r.add(OpKind{"unary_mlp", &run_unary_mlp, nullptr, MK_OP_READS_X});
   r.add(OpKind{"state_space", &run_state_space, nullptr, MK_OP_READS_X});
   r.add(OpKind{"normed_sum", &run_normed_sum, &tiles_normed_sum, MK_OP_READS_X});
-  r.add(OpKind{"keep_stream", &run_keep_stream, nullptr, MK_OP_KEPT_STREAM});
-  r.add(OpKind{"stream_mix", &run_stream_mix, nullptr, MK_OP_KEPT_STREAM});
+  r.add(OpKind{"keep_stream", &run_keep_stream, nullptr, MK_OP_KEPT_STREAM | MK_OP_FOLDS_PENDING});
+  r.add(OpKind{"stream_mix", &run_stream_mix, nullptr, MK_OP_KEPT_STREAM | MK_OP_FOLDS_PENDING});
   r.add(OpKind{"head", &run_head, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
   r.fixed_stream_tokens = &fixed_stream_tokens;
 }

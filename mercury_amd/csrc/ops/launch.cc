@@ -429,10 +429,11 @@ void unary_mlp(Launch& l, const void* x, int m, int hidden, const void* w_up, co
                int inter, int act, float* h, const float*& pending, int& pending_count) {
   pending = nullptr;
   pending_count = 0;
-  void* up = linear(l, x, m, w_up, inter, hidden, nullptr, kF32, nullptr, l.dtype(), false);
+  // the product in float32, so that the activation's result is rounded once
+  void* up = linear(l, x, m, w_up, inter, hidden, nullptr, kF32, nullptr, kF32, false);
   void* acted = l.alloc((size_t)m * inter * l.elem());
   if (!l.dry() && m > 0) {
-    check_core(need_core().mk_unary_act(up, acted, l.dtype(), (long long)m * inter, act,
+    check_core(need_core().mk_unary_act(up, kF32, acted, l.dtype(), (long long)m * inter, act,
                                         l.stream()), "unary_act");
   }
   project_into_stream(l, acted, m, w_down, hidden, inter, nullptr, kF32, h, pending,
