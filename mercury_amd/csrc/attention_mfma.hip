@@ -59,6 +59,14 @@ struct AttnParams {
   int tile_rows;     // rows per tile: 16, 32 or 64
   int kv_fold;       // key/value heads per workgroup of the unstaged kernel: 1, 2 or 4
   int direct;        // no tile list: tile t is the one new token of sequence t
+  // A bound on the scaled score, cap * tanh(scaled / cap), as two factors for the raw score:
+  // raw' = cap_out * tanh(raw * cap_in) with cap_in = scale / cap, cap_out = cap / scale, so
+  // that everything behind it works on raw' as it does on raw.  cap_in 0: no bound.
+  float cap_in, cap_out;
+  // [query heads], or null: exp(sinks[head]) stands once more in the softmax's denominator
+  // (an extra key of that score whose value is zero; the part that holds the first keys
+  // carries it).
+  const float* sinks;
 };
 
 #define ATTN_WAVES 4
@@ -206,9 +214,10 @@ struct TileState {
 // With it product h takes keys q * 8 + h * 4 + m (q, m = 0..3), and a lane holds the eight
 // consecutive keys g4 * 8 + 0..7: its operand of the second product is then one 16-byte
 // piece of a row of values.
-template <int D, int RT, bool MASKED, bool PERM>
+template <int D, int RT, bool MASKED, bool PERM, bool CAP = false>
 __device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBlock<D>& blk,
-                                             int key0, float c, int g4) {
+                                             int key0, float c, int g4, float cap_in = 0.f,
+                                             float cap_out = 0.f) {
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     float s[8];
@@ -221,6 +230,12 @@ __device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBloc
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float v = sc[i];
+        if (CAP) {
+          // tanh(x) = 1 - 2 / (1 + e^(2x)), the exponential and the quotient by the hardware's
+          // own instructions; cap_in carries the 2 log2(e)
+          const float e2 = __builtin_amdgcn_exp2f(v * cap_in);
+          v = cap_out * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e2));
+        }
         if (MASKED) {
           const int key = key0 + (PERM ? g4 * 8 + h * 4 + i : h * 16 + g4 * 4 + i);
           const bool ok = blk.live[h] && st.row_ok[t] && key <= st.pos[t] && key >= st.lo[t];
@@ -262,13 +277,14 @@ __device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBloc
 }
 
 // Blocks wholly inside what every row of the tiles sees take the unmasked path.
-template <int D, int RT, bool PERM = false>
+template <int D, int RT, bool PERM = false, bool CAP = false>
 __device__ __forceinline__ void attend(TileState<D, RT>& st, const KeyBlock<D>& blk, int key0,
-                                       float c, int g4, int all_see_upto, int all_see_from) {
+                                       float c, int g4, int all_see_upto, int all_see_from,
+                                       float cap_in = 0.f, float cap_out = 0.f) {
   if (key0 + 31 <= all_see_upto && key0 >= all_see_from)
-    attend_block<D, RT, false, PERM>(st, blk, key0, c, g4);
+    attend_block<D, RT, false, PERM, CAP>(st, blk, key0, c, g4, cap_in, cap_out);
   else
-    attend_block<D, RT, true, PERM>(st, blk, key0, c, g4);
+    attend_block<D, RT, true, PERM, CAP>(st, blk, key0, c, g4, cap_in, cap_out);
 }
 
 // RT: 16-row tiles per wavefront.  A decoded token's heads fill one tile (RT = 1, and the
@@ -291,7 +307,7 @@ __device__ __forceinline__ void attend(TileState<D, RT>& st, const KeyBlock<D>& 
 // before the first product instead of four, and parts that are equal for every sequence
 // whatever its length.  (A first block past a sequence's end is read from whatever page the
 // table names there, which exists, and masked.)
-template <int D, int RT, int AHEAD, bool GROUPED = false, bool DIRECT = false>
+template <int D, int RT, int AHEAD, bool GROUPED = false, bool DIRECT = false, bool CAP = false>
 __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) void attn_mfma_kernel(AttnParams p) {
   static_assert(!GROUPED || (RT == 1 && D <= 128), "grouped parts: one tile, heads up to 128");
   static_assert(!DIRECT || (RT == 1 && AHEAD == 1), "direct: one tile, one block ahead");
@@ -361,12 +377,13 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
   const int see_upto = pos0 + row0 / G;
   const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
   const float c = p.scale * 1.44269504088896340736f;
+  const float cap_in = CAP ? p.cap_in * 2.88539008177792681472f : 0.f, cap_out = p.cap_out;
 
   if (AHEAD == 0) {
     KeyBlock<D> blk;
     for (int b = b0; b < b1; ++b) {
       load_key_block<D>(blk, p, tw, b, b1, kmin, kmax, kvh, lane);
-      attend<D, RT>(st, blk, b << 5, c, g4, see_upto, see_from);
+      attend<D, RT, false, CAP>(st, blk, b << 5, c, g4, see_upto, see_from, cap_in, cap_out);
     }
   } else if (AHEAD == 1) {
     KeyBlock<D> x, y;
@@ -378,22 +395,22 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
         const bool more = b + splits < blk_hi;
         sp.pages(more ? j + 1 : j, p.page_shift, lane, page_lo, page_hi);
         load_key_block_at<D>(y, p, b + splits, page_lo, page_hi, more, kvh, lane);
-        attend<D, RT>(st, x, b << 5, c, g4, see_upto, see_from);
+        attend<D, RT, false, CAP>(st, x, b << 5, c, g4, see_upto, see_from, cap_in, cap_out);
         if (more) {
           const bool further = b + 2 * splits < blk_hi;
           sp.pages(further ? j + 2 : j + 1, p.page_shift, lane, page_lo, page_hi);
           load_key_block_at<D>(x, p, b + 2 * splits, page_lo, page_hi, further, kvh, lane);
-          attend<D, RT>(st, y, (b + splits) << 5, c, g4, see_upto, see_from);
+          attend<D, RT, false, CAP>(st, y, (b + splits) << 5, c, g4, see_upto, see_from, cap_in, cap_out);
         }
       }
     } else {
     load_key_block<D>(x, p, tw, b0, b1, kmin, kmax, kvh, lane);
     for (int b = b0; b < b1; b += 2) {
       load_key_block<D>(y, p, tw, b + 1, b1, kmin, kmax, kvh, lane);
-      attend<D, RT>(st, x, b << 5, c, g4, see_upto, see_from);
+      attend<D, RT, false, CAP>(st, x, b << 5, c, g4, see_upto, see_from, cap_in, cap_out);
       if (b + 1 < b1) {
         load_key_block<D>(x, p, tw, b + 2, b1, kmin, kmax, kvh, lane);
-        attend<D, RT>(st, y, (b + 1) << 5, c, g4, see_upto, see_from);
+        attend<D, RT, false, CAP>(st, y, (b + 1) << 5, c, g4, see_upto, see_from, cap_in, cap_out);
       }
     }
     }
@@ -403,14 +420,14 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
     load_key_block<D>(y, p, tw, b0 + 1, b1, kmin, kmax, kvh, lane);
     for (int b = b0; b < b1; b += 3) {
       load_key_block<D>(z, p, tw, b + 2, b1, kmin, kmax, kvh, lane);
-      attend<D, RT>(st, x, b << 5, c, g4, see_upto, see_from);
+      attend<D, RT, false, CAP>(st, x, b << 5, c, g4, see_upto, see_from, cap_in, cap_out);
       if (b + 1 < b1) {
         load_key_block<D>(x, p, tw, b + 3, b1, kmin, kmax, kvh, lane);
-        attend<D, RT>(st, y, (b + 1) << 5, c, g4, see_upto, see_from);
+        attend<D, RT, false, CAP>(st, y, (b + 1) << 5, c, g4, see_upto, see_from, cap_in, cap_out);
       }
       if (b + 2 < b1) {
         load_key_block<D>(y, p, tw, b + 4, b1, kmin, kmax, kvh, lane);
-        attend<D, RT>(st, z, (b + 2) << 5, c, g4, see_upto, see_from);
+        attend<D, RT, false, CAP>(st, z, (b + 2) << 5, c, g4, see_upto, see_from, cap_in, cap_out);
       }
     }
   }
@@ -455,6 +472,15 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
         o.z += v.z * wt;
         o.w += v.w * wt;
       }
+      if (p.sinks && blockIdx.z == 0) {
+        // the sink as one more key of the first part, its value zero
+        const float sink = p.sinks[kvh * G + flat % G] * 1.44269504088896340736f;
+        const float m_new = fmaxf(mx, sink);
+        const float keep = mx == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mx - m_new);
+        total = total * keep + __builtin_amdgcn_exp2f(sink - m_new);
+        o.x *= keep, o.y *= keep, o.z *= keep, o.w *= keep;
+        mx = m_new;
+      }
       if (p.num_splits == 1) {
         const float inv = total > 0.f ? 1.f / total : 0.f;
         bf16_t* dst = p.out + (size_t)(q0 + flat / G) * p.out_stride + (kvh * G + flat % G) * D + dim;
@@ -476,6 +502,16 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
     float l = st.lsum[t];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
+    if (p.sinks && split == 0) {
+      // the sink as one more key of the first part, its value zero
+      const float sink = p.sinks[head[t]] * 1.44269504088896340736f;
+      const float m_new = fmaxf(st.m[t], sink);
+      const float keep = st.m[t] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(st.m[t] - m_new);
+      l = l * keep + __builtin_amdgcn_exp2f(sink - m_new);
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) st.acc[t][dt] *= keep;
+      st.m[t] = m_new;
+    }
     // acc[t][dt][i] is O^T[dim = dt*16 + g4*4 + i][row r of tile t].
     if (p.num_splits == 1) {
       if (!st.row_ok[t]) continue;
@@ -1347,8 +1383,34 @@ static void launch_merge(const AttnParams& p, hipStream_t stream) {
   }
 }
 
+// The instantiations that bound the score: tiles of 16 rows only.
+template <int D>
+static void launch_attn_capped(const AttnParams& p, bool merge, hipStream_t stream) {
+  if constexpr (D <= 128) {
+    if (attn_grouped(16, p.num_splits)) {
+      AttnParams g = p;
+      g.num_splits = p.num_splits / ATTN_WAVES;
+      const dim3 grid(g.num_tiles, g.n_kv, g.num_splits);
+      if (g.direct) attn_mfma_kernel<D, 1, ATTN_AHEAD_16, true, true, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(g);
+      else attn_mfma_kernel<D, 1, ATTN_AHEAD_16, true, false, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(g);
+      if (merge) launch_merge<D>(g, stream);
+      return;
+    }
+  }
+  const int per = ATTN_WAVES / p.kv_fold;   // tiles per workgroup
+  dim3 grid((p.num_tiles + per - 1) / per, p.n_kv / p.kv_fold, p.num_splits);
+  const int threads = 64 * ATTN_WAVES;
+  if (p.direct) attn_mfma_kernel<D, 1, ATTN_AHEAD_16, false, true, true><<<grid, threads, 0, stream>>>(p);
+  else attn_mfma_kernel<D, 1, ATTN_AHEAD_16, false, false, true><<<grid, threads, 0, stream>>>(p);
+  if (merge) launch_merge<D>(p, stream);
+}
+
 template <int D>
 static void launch_attn(const AttnParams& p, int rows_per_tile, bool merge, hipStream_t stream) {
+  if (p.cap_in != 0.f) {
+    launch_attn_capped<D>(p, merge, stream);
+    return;
+  }
   if constexpr (D <= 128) {
     if (attn_grouped(rows_per_tile, p.num_splits)) {
       AttnParams g = p;
@@ -1491,7 +1553,11 @@ static int attention_mfma(const void* q, int q_stride, void* out, int out_stride
                           const int* block_table, int table_stride, int page_size, int n_q,
                           int n_kv, int d, float scale, int window, int rows_per_tile, int staged,
                           int num_splits, int split_blocks, float* part_o, float* part_ml,
-                          bool merge, hipStream_t stream) {
+                          bool merge, hipStream_t stream, float score_cap = 0.f,
+                          const float* sinks = nullptr) {
+  MK_REQUIRE(score_cap >= 0.f, "attention: negative score cap");
+  MK_REQUIRE((score_cap == 0.f && sinks == nullptr) || (rows_per_tile == 16 && staged == 0),
+             "attention: a bounded score or sinks run in tiles of 16 rows, keys unstaged");
   if (int code = mk_attention_mfma_check(q_stride, out_stride, num_tiles, page_size, n_q, n_kv, d,
                                          scale, window, rows_per_tile, staged, num_splits,
                                          split_blocks, part_o && part_ml)) {
@@ -1534,6 +1600,9 @@ static int attention_mfma(const void* q, int q_stride, void* out, int out_stride
   // of 8 key/value heads: 10 us unfolded, 16 folded; 64 tokens: 194 and 186)
   p.kv_fold = num_tiles < 32 ? 1 : (n_kv % 4 == 0 ? 4 : (n_kv % 2 == 0 ? 2 : 1));
   p.direct = direct;
+  p.cap_in = score_cap > 0.f ? scale / score_cap : 0.f;
+  p.cap_out = score_cap > 0.f ? score_cap / scale : 0.f;
+  p.sinks = sinks;
   if (staged >= 8) {
     if (d == 64) launch_wide<64>(p, staged, stream); else launch_wide<128>(p, staged, stream);
     MK_LAUNCH_CHECK("attention_mfma");
@@ -1562,6 +1631,21 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
                         num_tiles, cu_q, kv_len, block_table, table_stride, page_size, n_q, n_kv, d,
                         scale, window, rows_per_tile, staged, num_splits, split_blocks, part_o,
                         part_ml, true, stream);
+}
+
+extern "C" int mk_attention_mfma_scored(const void* q, int q_stride, void* out, int out_stride,
+                                        const void* k_cache, const void* v_cache,
+                                        const int* tile_seq, const int* tile_row0, int num_tiles,
+                                        const int* cu_q, const int* kv_len,
+                                        const int* block_table, int table_stride, int page_size,
+                                        int n_q, int n_kv, int d, float scale, int window,
+                                        int num_splits, int split_blocks, float score_cap,
+                                        const float* sinks, float* part_o, float* part_ml,
+                                        hipStream_t stream) {
+  return attention_mfma(q, q_stride, out, out_stride, k_cache, v_cache, tile_seq, tile_row0,
+                        num_tiles, cu_q, kv_len, block_table, table_stride, page_size, n_q, n_kv, d,
+                        scale, window, 16, 0, num_splits, split_blocks, part_o, part_ml, true,
+                        stream, score_cap, sinks);
 }
 
 extern "C" int mk_attention_mfma_parts_written(int rows_per_tile, int num_splits, int d) {

@@ -97,6 +97,8 @@ AttendArgs attend_from(const py::dict& d) {
   a.v_cache = ptr_of<const void>(d, "v_cache");
   a.score_cap = get<float>(d, "score_cap", 0.f);
   a.distance_slopes = ptr_of<const float>(d, "distance_slopes");
+  a.sinks = ptr_of<const float>(d, "sinks");
+  a.value_dim = get<int>(d, "value_dim", 0);
   return a;
 }
 

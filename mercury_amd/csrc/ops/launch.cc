@@ -262,9 +262,9 @@ Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, c
 
 AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
                        const AttendForce& force) {
-  if (!a.plain_scores()) {
+  if (a.distance_slopes != nullptr) {
     if (force.kernel == 2) {
-      throw KernelError("attention: the matrix-core kernels neither cap nor bias the score");
+      throw KernelError("attention: the matrix-core kernels do not bias the score by distance");
     }
     return AttentionPlan();     // the float32-arithmetic kernel
   }
@@ -275,6 +275,17 @@ AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
     return AttentionPlan();
   }
   const std::vector<int> counts(step.counts, step.counts + step.num_seqs);
+  if (!a.plain_scores()) {
+    // a bounded score or sinks: the matrix-core kernel of 16-row tiles, keys unstaged
+    if (force.tile_rows > 16 || force.staged > 0) {
+      throw KernelError("attention: a bounded score or sinks run in tiles of 16 rows, unstaged");
+    }
+    // (decoding: the planner's own choice is 16 rows, and only then may it drop the tile list)
+    const int rows = step.max_q_len == 1 && a.n_q / a.n_kv <= 16 && force.tile_rows <= 0 ? -1 : 16;
+    return plan_attention(dtype, a.head_dim, a.page_size, a.n_q, a.n_kv, a.window, counts,
+                          step.max_q_len, step.max_kv_len, force.kernel, rows, 0, force.splits,
+                          force.split_blocks);
+  }
   return plan_attention(dtype, a.head_dim, a.page_size, a.n_q, a.n_kv, a.window, counts,
                         step.max_q_len, step.max_kv_len, force.kernel, force.tile_rows, force.staged,
                         force.splits, force.split_blocks);
@@ -314,6 +325,15 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
   }
   if (l.dry() || m == 0) return out;
   const mk_tile_list& tiles = tiles_for(step, a.n_q / a.n_kv, plan.tile_rows);
+  if (!a.plain_scores()) {
+    check_mfma(need_mfma().mk_attention_mfma_scored(
+                   q.q, q.stride, out, a.n_q * d, a.k_cache, a.v_cache,
+                   plan.direct ? nullptr : tiles.seq, plan.direct ? nullptr : tiles.row0,
+                   tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride, a.page_size, a.n_q,
+                   a.n_kv, d, a.scale, a.window, plan.splits, plan.split_blocks, a.score_cap,
+                   a.sinks, part_o, part_ml, l.stream()), "attention");
+    return out;
+  }
   check_mfma(need_mfma().mk_attention_mfma(
                  q.q, q.stride, out, a.n_q * d, a.k_cache, a.v_cache,
                  plan.direct ? nullptr : tiles.seq, plan.direct ? nullptr : tiles.row0,
@@ -343,7 +363,7 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
   int heads_per_slice = 0, written = 0;
   bool wide = false;
   const bool fixed = h_fixed != nullptr || (l.dry() && l.ctx->stream_fixed);
-  if (fold != 0 && plan.mfma && plan.splits > 1 && !plan.staged && plan.rows == 16 &&
+  if (fold != 0 && plan.mfma && a.plain_scores() && plan.splits > 1 && !plan.staged && plan.rows == 16 &&
       step.max_q_len == 1 && plan.num_tiles == m && !b_o && a.n_q / a.n_kv <= 16) {
     const KernelTable& t = need_mfma();
     written = t.mk_attention_mfma_parts_written(plan.rows, plan.splits, d);

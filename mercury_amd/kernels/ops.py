@@ -490,7 +490,8 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
               kernel: str = "auto", tile_rows: int | None = None,
               split_override: tuple | None = None, staged: bool | None = None,
               score_cap: float | None = None,
-              distance_slopes: torch.Tensor | None = None) -> torch.Tensor:
+              distance_slopes: torch.Tensor | None = None,
+              sinks: torch.Tensor | None = None) -> torch.Tensor:
     """Causal grouped-query attention of every token of the step over its sequence's cached
     keys; q is read from rows of `q` with stride `q_stride` (the fused qkv buffer).
     `step` describes the batch (positions, token_seq, cu_q, kv_len, spans, tiles());
@@ -504,10 +505,15 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     whether workgroups of four wavefronts share the keys and values of one sequence's rows
     through LDS; by default the step's size decides all three.
     score_cap bounds the scaled score to cap * tanh(score / cap); distance_slopes (float32
-    [n_q]) subtracts slope[head] * (query position - key position) from it.  With either the
-    float32-arithmetic kernel runs, whatever the dtype.
+    [n_q]) subtracts slope[head] * (query position - key position) from it; sinks (float32
+    [n_q]) adds exp(sink[head]) once to the softmax's denominator.  With a distance penalty
+    the float32-arithmetic kernel runs, whatever the dtype; a bounded score and sinks also run
+    on the matrix cores, in tiles of 16 rows.
     """
-    _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out, distance_slopes)
+    _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out, distance_slopes,
+         sinks)
+    if sinks is not None and (sinks.dtype != torch.float32 or sinks.shape != (n_q,)):
+        raise KernelArgumentError(f"attention: sinks must be float32 [{n_q}]")
     if distance_slopes is not None and (distance_slopes.dtype != torch.float32
                                         or distance_slopes.shape != (n_q,)):
         raise KernelArgumentError(f"attention: distance_slopes must be float32 [{n_q}]")
@@ -528,7 +534,7 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     args = dict(n_q=n_q, n_kv=n_kv, head_dim=head_dim, page_size=page_size,
                 window=int(window or 0), scale=float(scale), k_cache=_ptr(k_cache),
                 v_cache=_ptr(v_cache), score_cap=float(score_cap or 0.0),
-                distance_slopes=_ptr(distance_slopes))
+                distance_slopes=_ptr(distance_slopes), sinks=_ptr(sinks))
 
     def tiles(group, rows):
         seq, row0, count = step.tiles(group, rows)

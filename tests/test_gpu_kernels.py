@@ -993,7 +993,7 @@ def test_attention_with_a_capped_score_and_a_distance_penalty(dtype, cap, with_s
     """What the reference's attention does not have and another mixer may want: the score
     bounded by cap * tanh(. / cap), and slope[head] * distance subtracted from it (a position
     encoding that lives in the score).  The float32-arithmetic kernel computes both, in
-    either dtype; the matrix-core kernel refuses them."""
+    either dtype; the matrix-core kernel bounds the score too and refuses the penalty."""
     n_q, n_kv, d, page = 6, 2, 32, 16
     lens = [70, 33, 5]
     slopes = torch.tensor([0.5 ** (i + 1) for i in range(n_q)]) if with_slopes else None
@@ -1023,9 +1023,13 @@ def test_attention_with_a_capped_score_and_a_distance_penalty(dtype, cap, with_s
     # the terms matter: without them the result is another
     bare = ops().attention(*args).float().cpu().view(-1, n_q, d)
     assert float((bare - want).abs().max()) > 10 * tol(dtype)["atol"]
-    if dtype == torch.bfloat16:
-        with pytest.raises(RuntimeError, match="neither cap nor bias"):
-            ops().attention(*args, score_cap=cap or 1.0, kernel="mfma")
+    if dtype == torch.bfloat16 and slopes is not None:
+        with pytest.raises(RuntimeError, match="do not bias the score by distance"):
+            ops().attention(*args, score_cap=cap, distance_slopes=slopes.to(DEV), kernel="mfma")
+    elif dtype == torch.bfloat16:
+        # a bounded score alone also runs on the matrix cores
+        fast = ops().attention(*args, score_cap=cap, kernel="mfma")
+        torch.testing.assert_close(fast.float().cpu().view(-1, n_q, d), want, **tol(dtype))
 
 
 def test_attention_gqa_equals_mha_with_repeated_heads():
