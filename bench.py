@@ -23,7 +23,13 @@ times the prompt attention kernel alone at the models' head shapes, and
 times prompts of 2,048 tokens and decode steps (batch 8, context 4,096) of the Talolorn design
 (latent attention, parallel blocks; once with dense feed-forwards, once with routed experts)
 at two sets of layer sizes, beside a Qwen2 model of the same width, depth, heads and
-feed-forward size, and
+feed-forward size;
+
+    python bench.py --larozen [--larozen-only NAME]
+
+does the same for the Larozen design (rotated attention with a bounded score whose values are
+its keys, alternating with layers of a sink attention beside a state-space mixer; squared-relu
+feed-forwards; one re-entry of the stream), and
 
     python bench.py --shape 32b --serve
 
@@ -98,6 +104,11 @@ def parse_args(argv=None):
                         "Talolorn design at two sets of layer sizes, beside a Qwen2 model of equal size")
     p.add_argument("--talolorn-only", default=None,
                    help="run one entry of the comparison only (e.g. small/talolorn-moe), for a profiler")
+    p.add_argument("--larozen", action="store_true",
+                   help="prompts and decode steps of the Larozen design at two sets of layer "
+                        "sizes, beside Qwen2 at equal width, depth, heads and feed-forward size")
+    p.add_argument("--larozen-only", default=None,
+                   help="run one entry of the comparison only (e.g. small/larozen), for a profiler")
     p.add_argument("--serve-requests", type=int, default=64)
     p.add_argument("--serve-chunk", type=int, default=512)
     return p.parse_args(argv)
@@ -423,14 +434,58 @@ def talolorn_configs(z: dict) -> dict:
     }
 
 
+# Layer sizes for `--larozen`: four layers (attention, side by side, attention, side by side; the
+# stream re-enters before the third), a state-space mixer twice the width inside with heads of
+# 64 columns and 128 rows of state.
+LAROZEN_SIZES = {
+    "small": dict(width=2048, heads=16, kv_heads=4, dim=128, ss_heads=64, ss_vdim=64, state=128,
+                  groups=4, ff=8192, vocab=32000, layers=4),
+    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, ss_heads=128, ss_vdim=64, state=128,
+                  groups=8, ff=12288, vocab=32000, layers=4),
+}
+
+
+def larozen_configs(z: dict) -> dict:
+    """name -> config.json of the two models compared at the sizes `z`."""
+    scale = z["dim"] ** -0.5
+    attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                 "scale": scale, "softcap": 30.0, "rot": {"base": 10000.0, "dims": z["dim"] // 2}}
+    left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+            "scale": scale, "q_temp": {"coef": 0.5, "every": 256}}
+    right = {"heads": z["ss_heads"], "vdim": z["ss_vdim"], "state": z["state"], "groups": z["groups"],
+             "conv": 4, "norm_groups": z["groups"]}
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    pair = [{"type": "attention", "mixer": attention, "mlp": mlp},
+            {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp}]
+    return {
+        "larozen": {"architecture": "Larozen", "vocab": z["vocab"], "width": z["width"],
+                    "norm": {"eps": 1e-6}, "layers": pair * (z["layers"] // 2),
+                    "loop": {"start": 2, "stop": z["layers"], "times": 1}},
+        "qwen2": {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+                  "hidden_size": z["width"], "intermediate_size": z["ff"],
+                  "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+                  "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
+                  "vocab_size": z["vocab"], "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
+                  "tie_word_embeddings": True, "max_position_embeddings": 32768},
+    }
+
+
 def talolorn_main(args) -> int:
+    return compare_main(args, "Talolorn", TALOLORN_SIZES, talolorn_configs, args.talolorn_only)
+
+
+def larozen_main(args) -> int:
+    return compare_main(args, "Larozen", LAROZEN_SIZES, larozen_configs, args.larozen_only)
+
+
+def compare_main(args, design: str, sizes: dict, configs, only) -> int:
     import torch
 
     rows = {}
-    for size, z in TALOLORN_SIZES.items():
-        for name, cfg in talolorn_configs(z).items():
+    for size, z in sizes.items():
+        for name, cfg in configs(z).items():
             key = f"{size}/{name}"
-            if args.talolorn_only and args.talolorn_only != key:
+            if only and only != key:
                 continue
             bench = Bench(cfg, args.dtype, args.batch, args.context, args.seed, not args.no_lookahead)
             run = bench.decode(args.batch, args.context, args.steps, args.warmup)
@@ -448,10 +503,10 @@ def talolorn_main(args) -> int:
             torch.cuda.empty_cache()
     print(json.dumps({
         "metric": f"decode tok/s at batch {args.batch}, context {args.context}, and tok/s of a "
-                  f"{PREFILL_TOKENS}-token prompt: Talolorn beside Qwen2 at equal sizes",
+                  f"{PREFILL_TOKENS}-token prompt: {design} beside Qwen2 at equal sizes",
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-        "sizes": TALOLORN_SIZES, "rows": rows}))
+        "sizes": sizes, "rows": rows}))
     return 0
 
 
@@ -465,6 +520,8 @@ def main(argv=None) -> int:
         return attention_main(args)
     if args.talolorn:
         return talolorn_main(args)
+    if args.larozen:
+        return larozen_main(args)
     model_name, shape = SHAPES[args.shape]
     cfg = dict(shape)
     full_layers = cfg["num_hidden_layers"]

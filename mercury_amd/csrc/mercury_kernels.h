@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 27
+#define MK_ABI_VERSION 28
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
@@ -250,7 +250,12 @@ int mk_ssm_scan(const float* xbc, int xbc_stride, const float* proj, int proj_st
                 int dt_col, const void* dt_bias, const void* a_log, const void* d_skip,
                 int weight_dtype, float* state, long long slot_stride, const int* slots,
                 const int* cu_q, int heads, int P, int N, int groups, float* y_out, int tokens,
-                int num_seqs, hipStream_t stream);
+                int num_seqs, int total_chunks, float* workspace, hipStream_t stream);
+// A step with a sequence of more than mk_ssm_chunk_tokens() tokens runs the recurrence in
+// chunks side by side: total_chunks is then the sum over the sequences of ceil(tokens /
+// chunk), `workspace` mk_ssm_scan_workspace(...) floats of scratch memory; else 0 and null.
+int mk_ssm_chunk_tokens();
+long long mk_ssm_scan_workspace(int total_chunks, int heads, int P, int N);
 long long mk_ssm_state_floats(int heads, int P, int N);
 // out[t, part] = y[t, part] / rms(y[t, part]) * weight[part], the row in `parts` equal parts.
 int mk_group_rmsnorm(const float* y, void* out, int dtype, const void* weight, int weight_dtype,

@@ -470,6 +470,21 @@ void state_space(Launch& l, const void* x, int m, int hidden, const StateSpaceAr
   float* xbc = (float*)l.alloc((size_t)m * channels * 4);
   float* y = (float*)l.alloc((size_t)m * inner * 4);
   void* normed = l.alloc((size_t)m * inner * l.elem());
+  // a step with a sequence longer than a chunk runs the recurrence in chunks side by side
+  const KernelTable& core = need_core();
+  const int chunk = core.mk_ssm_chunk_tokens();
+  int total_chunks = 0, longest = 0;
+  for (int i = 0; i < step.num_seqs; ++i) {
+    total_chunks += (step.counts[i] + chunk - 1) / chunk;
+    longest = std::max(longest, step.counts[i]);
+  }
+  if (longest <= chunk) total_chunks = 0;
+  float* scan_ws = nullptr;
+  if (total_chunks) {
+    const long long floats = core.mk_ssm_scan_workspace(total_chunks, a.heads, a.vdim, a.state_size);
+    if (floats < 0) throw KernelError("state_space: the recurrence does not run these sizes");
+    scan_ws = (float*)l.alloc((size_t)floats * 4);
+  }
   if (!l.dry() && m > 0) {
     const KernelTable& t = need_core();
     if (!a.state) throw KernelError("state_space: no state tensor");
@@ -480,7 +495,7 @@ void state_space(Launch& l, const void* x, int m, int hidden, const StateSpaceAr
     check_core(t.mk_ssm_scan(xbc, channels, proj, width, 0, inner + channels, a.dt_bias, a.a_log,
                              a.d_skip, a.vector_dtype, a.state + a.carried_floats(), a.slot_floats,
                              step.state_slots, step.cu_q, a.heads, a.vdim, a.state_size, a.groups,
-                             y, m, step.num_seqs, l.stream()), "ssm_scan");
+                             y, m, step.num_seqs, total_chunks, scan_ws, l.stream()), "ssm_scan");
     check_core(t.mk_group_rmsnorm(y, normed, l.dtype(), a.norm, a.vector_dtype, a.eps, m, inner,
                                   a.norm_groups, l.stream()), "group_rmsnorm");
   }

@@ -83,16 +83,31 @@ __global__ void conv_carry_kernel(const float* __restrict__ proj, int row_stride
   }
 }
 
+// Long portions are cut into chunks of SS_CHUNK tokens that run side by side, in three passes:
+// every chunk's recurrence from a zero state, which leaves the chunk's own contribution to
+// the state at its end and the product of its decays (SS_LOCAL); one pass over the chunks of
+// a sequence in order, S_in(k + 1) = decay(k) S_in(k) + local(k), from the state the slot
+// holds, which leaves every chunk the state it starts from and the slot the last one
+// (ssm_combine_kernel); and every chunk's recurrence again from that state, now with its
+// outputs (SS_FROM).  Twice the arithmetic, for as many workgroups as there are chunks
+// instead of one chain of dependent steps as long as the portion.  A step whose sequences all
+// bring at most SS_CHUNK tokens (decoding) runs the recurrence once, slot to slot (SS_DIRECT).
+enum { SS_DIRECT = 0, SS_LOCAL = 1, SS_FROM = 2 };
+#define SS_CHUNK 128
+
+__device__ __forceinline__ int chunks_of(int tokens) { return (tokens + SS_CHUNK - 1) / SS_CHUNK; }
+
 // lane -> (column within the wavefront's 8, slice of n); entry i of a lane is
 // n = (i / 4) * 32 + slice * 4 + i % 4, so that four entries are one 16-byte LDS read and the
 // eight slices read 128 contiguous bytes.
-template <int NI, typename TW>
+template <int NI, typename TW, int MODE>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(
     const float* __restrict__ xbc, int xbc_stride, const float* __restrict__ proj,
     int proj_stride, int z_col, int dt_col, const void* __restrict__ dt_bias,
     const void* __restrict__ a_log, const void* __restrict__ d_skip, float* __restrict__ state,
     size_t slot_stride, const int* __restrict__ slots, const int* __restrict__ cu_q, int heads,
-    int P, int N, int groups, float* __restrict__ y_out) {
+    int P, int N, int groups, float* __restrict__ y_out, float* __restrict__ chunk_state,
+    size_t chunk_stride, float* __restrict__ chunk_decay) {
   constexpr int NPAD = NI * 8;
   __shared__ __attribute__((aligned(16))) float sB[SS_TOKENS][NPAD];
   __shared__ __attribute__((aligned(16))) float sC[SS_TOKENS][NPAD];
@@ -100,25 +115,41 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
   __shared__ float sZ[SS_TOKENS][SS_COLS];
   __shared__ float sDt[SS_TOKENS], sDecay[SS_TOKENS];
 
-  const int seq = blockIdx.z, head = blockIdx.y, pblock = blockIdx.x;
+  const int head = blockIdx.y, pblock = blockIdx.x;
+  int seq = blockIdx.z, first, count;
+  if (MODE == SS_DIRECT) {
+    first = cu_q[seq];
+    count = cu_q[seq + 1] - first;
+  } else {
+    // chunk blockIdx.z of the step: the host launched as many as the sequences have together
+    int chunk = blockIdx.z;
+    seq = 0;
+    for (int n = chunks_of(cu_q[1] - cu_q[0]); chunk >= n; n = chunks_of(cu_q[seq + 1] - cu_q[seq])) {
+      chunk -= n;
+      ++seq;
+    }
+    first = cu_q[seq] + chunk * SS_CHUNK;
+    count = min(SS_CHUNK, cu_q[seq + 1] - first);
+  }
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int slice = lane >> 3, col_in_wave = lane & 7;
   const int col = pblock * SS_COLS + wave * 8 + col_in_wave;   // column p of the head
   const int group = head / (heads / groups);
   const int inner = heads * P;
-  const int first = cu_q[seq], count = cu_q[seq + 1] - first;
   const int blocks8 = (P + SS_COLS - 1) / SS_COLS * (SS_COLS / 8);   // whole workgroups
 
-  float* mine = state + (size_t)slots[seq] * slot_stride +
-                ((size_t)head * blocks8 + (size_t)pblock * 4 + wave) * NI * 64;
+  const size_t within = ((size_t)head * blocks8 + (size_t)pblock * 4 + wave) * NI * 64;
+  float* mine = MODE == SS_DIRECT ? state + (size_t)slots[seq] * slot_stride + within
+                                  : chunk_state + (size_t)blockIdx.z * chunk_stride + within;
   const bool live = pblock * SS_COLS + wave * 8 < P;    // the wavefront has columns at all
   float S[NI];
 #pragma unroll
-  for (int i = 0; i < NI; ++i) S[i] = live ? mine[i * 64 + lane] : 0.f;
+  for (int i = 0; i < NI; ++i) S[i] = (MODE != SS_LOCAL && live) ? mine[i * 64 + lane] : 0.f;
 
   const float rate = expf(weight_at<TW>(a_log, head));
   const float bias = weight_at<TW>(dt_bias, head);
   const float skip = weight_at<TW>(d_skip, head);
+  float dt_sum = 0.f;
 
   for (int t0 = 0; t0 < count; t0 += SS_TOKENS) {
     const int n_tok = min(SS_TOKENS, count - t0);
@@ -127,14 +158,14 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
       const int tt = idx / NPAD, n = idx - tt * NPAD;
       const float* row = xbc + (size_t)(first + t0 + tt) * xbc_stride + inner;
       sB[tt][n] = n < N ? row[group * N + n] : 0.f;
-      sC[tt][n] = n < N ? row[groups * N + group * N + n] : 0.f;
+      if (MODE != SS_LOCAL) sC[tt][n] = n < N ? row[groups * N + group * N + n] : 0.f;
     }
     for (int idx = tid; idx < n_tok * SS_COLS; idx += 256) {
       const int tt = idx / SS_COLS, c = idx - tt * SS_COLS;
       const int p = pblock * SS_COLS + c;
       const size_t tok = first + t0 + tt;
       sX[tt][c] = p < P ? xbc[tok * xbc_stride + head * P + p] : 0.f;
-      sZ[tt][c] = p < P ? proj[tok * proj_stride + z_col + head * P + p] : 0.f;
+      if (MODE != SS_LOCAL) sZ[tt][c] = p < P ? proj[tok * proj_stride + z_col + head * P + p] : 0.f;
     }
     if (tid < n_tok) {
       const float raw = proj[(size_t)(first + t0 + tid) * proj_stride + dt_col + head] + bias;
@@ -147,7 +178,21 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
     for (int tt = 0; tt < n_tok; ++tt) {
       const float x = sX[tt][wave * 8 + col_in_wave];
       const float dtx = sDt[tt] * x, decay = sDecay[tt];
-      float y = 0.f;
+      if (MODE == SS_LOCAL) {
+        dt_sum += sDt[tt];
+#pragma unroll
+        for (int i4 = 0; i4 < NI / 4; ++i4) {
+          const float4 b = *(const float4*)&sB[tt][i4 * 32 + slice * 4];
+          float* s = &S[i4 * 4];
+          s[0] = fmaf(decay, s[0], dtx * b.x);
+          s[1] = fmaf(decay, s[1], dtx * b.y);
+          s[2] = fmaf(decay, s[2], dtx * b.z);
+          s[3] = fmaf(decay, s[3], dtx * b.w);
+        }
+        continue;
+      }
+      // four sums side by side (entries i % 4), added up at the end: ((y0 + y1) + (y2 + y3))
+      float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
 #pragma unroll
       for (int i4 = 0; i4 < NI / 4; ++i4) {
         const float4 b = *(const float4*)&sB[tt][i4 * 32 + slice * 4];
@@ -157,11 +202,12 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
         s[1] = fmaf(decay, s[1], dtx * b.y);
         s[2] = fmaf(decay, s[2], dtx * b.z);
         s[3] = fmaf(decay, s[3], dtx * b.w);
-        y = fmaf(s[0], c.x, y);
-        y = fmaf(s[1], c.y, y);
-        y = fmaf(s[2], c.z, y);
-        y = fmaf(s[3], c.w, y);
+        y0 = fmaf(s[0], c.x, y0);
+        y1 = fmaf(s[1], c.y, y1);
+        y2 = fmaf(s[2], c.z, y2);
+        y3 = fmaf(s[3], c.w, y3);
       }
+      float y = (y0 + y1) + (y2 + y3);
       y += __shfl_xor(y, 8, MK_WAVE);
       y += __shfl_xor(y, 16, MK_WAVE);
       y += __shfl_xor(y, 32, MK_WAVE);
@@ -171,10 +217,38 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
       }
     }
   }
-  if (live) {
+  if (MODE != SS_FROM && live) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) mine[i * 64 + lane] = S[i];
   }
+  if (MODE == SS_LOCAL && pblock == 0 && tid == 0) {
+    chunk_decay[(size_t)blockIdx.z * heads + head] = expf(-rate * dt_sum);
+  }
+}
+
+// The chunks of a sequence in order: chunk k's buffer holds what the chunk adds to the state
+// and receives the state the chunk starts from; the slot receives the state after the last.
+__global__ void ssm_combine_kernel(float* __restrict__ state, size_t slot_stride,
+                                   const int* __restrict__ slots, const int* __restrict__ cu_q,
+                                   float* __restrict__ chunk_state, size_t chunk_stride,
+                                   const float* __restrict__ chunk_decay, int heads,
+                                   size_t per_head) {
+  const int seq = blockIdx.y;
+  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= per_head * heads) return;
+  const int head = (int)(e / per_head);
+  int chunk0 = 0;
+  for (int s = 0; s < seq; ++s) chunk0 += chunks_of(cu_q[s + 1] - cu_q[s]);
+  const int n = chunks_of(cu_q[seq + 1] - cu_q[seq]);
+  float* slot = state + (size_t)slots[seq] * slot_stride;
+  float run = slot[e];
+  for (int k = 0; k < n; ++k) {
+    float* at = chunk_state + (size_t)(chunk0 + k) * chunk_stride + e;
+    const float local = *at;
+    *at = run;
+    run = fmaf(chunk_decay[(size_t)(chunk0 + k) * heads + head], run, local);
+  }
+  slot[e] = run;
 }
 
 // One workgroup per (token, part): out = y / rms(part of y) * weight.
@@ -242,17 +316,26 @@ extern "C" int mk_causal_conv_silu(const float* proj, int row_stride, int col0, 
   return 0;
 }
 
+// Tokens a chunk of the recurrence holds: a step with a longer sequence runs in chunks, and
+// wants mk_ssm_scan_workspace floats of scratch memory for `total_chunks` of them.
+extern "C" int mk_ssm_chunk_tokens() { return SS_CHUNK; }
+extern "C" long long mk_ssm_scan_workspace(int total_chunks, int heads, int P, int N) {
+  const long long per = mk_ssm_state_floats(heads, P, N);
+  return per < 0 ? -1 : (long long)total_chunks * (per + heads);
+}
+
 extern "C" int mk_ssm_scan(const float* xbc, int xbc_stride, const float* proj, int proj_stride,
                            int z_col, int dt_col, const void* dt_bias, const void* a_log,
                            const void* d_skip, int weight_dtype, float* state,
                            long long slot_stride, const int* slots, const int* cu_q, int heads,
                            int P, int N, int groups, float* y_out, int tokens, int num_seqs,
-                           hipStream_t stream) {
+                           int total_chunks, float* workspace, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && num_seqs >= 0 && heads > 0 && P > 0 && N > 0 && groups > 0,
              "ssm_scan: bad sizes");
   MK_REQUIRE(heads % groups == 0, "ssm_scan: %d heads are not a multiple of %d groups", heads, groups);
   MK_REQUIRE(N <= SS_MAX_NI * 8, "ssm_scan: state size %d exceeds %d", N, SS_MAX_NI * 8);
-  MK_REQUIRE(slot_stride >= mk_ssm_state_floats(heads, P, N),
+  const long long state_floats = mk_ssm_state_floats(heads, P, N);
+  MK_REQUIRE(slot_stride >= state_floats,
              "ssm_scan: a slot of %lld floats does not hold the state", slot_stride);
   MK_REQUIRE(xbc_stride >= heads * P + 2 * groups * N, "ssm_scan: x, B, C outside the row");
   MK_REQUIRE(z_col >= 0 && dt_col >= 0 && proj_stride >= z_col + heads * P &&
@@ -260,26 +343,54 @@ extern "C" int mk_ssm_scan(const float* xbc, int xbc_stride, const float* proj, 
   MK_REQUIRE(heads <= 65535 && num_seqs <= 65535, "ssm_scan: too many heads or sequences");
   MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "ssm_scan: weight dtype %d",
              weight_dtype);
+  // total_chunks 0: every sequence brings at most a chunk's tokens, one pass slot to slot;
+  // else the sum over the sequences of ceil(tokens / chunk), which the caller knows
+  MK_REQUIRE(total_chunks == 0 || (total_chunks >= num_seqs && total_chunks <= 65535 && workspace &&
+                                   (long long)total_chunks * SS_CHUNK >= tokens),
+             "ssm_scan: %d chunks for %d tokens of %d sequences (or no workspace)", total_chunks,
+             tokens, num_seqs);
+  MK_REQUIRE(total_chunks != 0 || (long long)num_seqs * SS_CHUNK >= tokens,
+             "ssm_scan: a sequence longer than a chunk runs in chunks");
   if (tokens == 0 || num_seqs == 0) return 0;
-  const dim3 grid((P + SS_COLS - 1) / SS_COLS, heads, num_seqs);
+  const int pblocks = (P + SS_COLS - 1) / SS_COLS;
   const int ni = entries_for(N);
-#define SS_LAUNCH(NI)                                                                          \
-  do {                                                                                         \
-    if (weight_dtype == MK_F32)                                                                \
-      ssm_scan_kernel<NI, float><<<grid, 256, 0, stream>>>(                                    \
-          xbc, xbc_stride, proj, proj_stride, z_col, dt_col, dt_bias, a_log, d_skip, state,    \
-          (size_t)slot_stride, slots, cu_q, heads, P, N, groups, y_out);                       \
-    else                                                                                       \
-      ssm_scan_kernel<NI, bf16_t><<<grid, 256, 0, stream>>>(                                   \
-          xbc, xbc_stride, proj, proj_stride, z_col, dt_col, dt_bias, a_log, d_skip, state,    \
-          (size_t)slot_stride, slots, cu_q, heads, P, N, groups, y_out);                       \
+  float* chunk_state = workspace;
+  float* chunk_decay = workspace ? workspace + (size_t)total_chunks * state_floats : nullptr;
+#define SS_RUN(NI, TW, MODE, grid)                                                              \
+  ssm_scan_kernel<NI, TW, MODE><<<grid, 256, 0, stream>>>(                                       \
+      xbc, xbc_stride, proj, proj_stride, z_col, dt_col, dt_bias, a_log, d_skip, state,         \
+      (size_t)slot_stride, slots, cu_q, heads, P, N, groups, y_out, chunk_state,                \
+      (size_t)state_floats, chunk_decay)
+#define SS_MODE(NI, MODE, grid)                                                                  \
+  do {                                                                                          \
+    if (weight_dtype == MK_F32) SS_RUN(NI, float, MODE, grid); else SS_RUN(NI, bf16_t, MODE, grid); \
   } while (0)
-  if (ni == 4) SS_LAUNCH(4);
-  else if (ni == 8) SS_LAUNCH(8);
-  else if (ni == 16) SS_LAUNCH(16);
-  else SS_LAUNCH(32);
+#define SS_LAUNCH(MODE, grid)                                                                    \
+  do {                                                                                          \
+    if (ni == 4) SS_MODE(4, MODE, grid);                                                         \
+    else if (ni == 8) SS_MODE(8, MODE, grid);                                                    \
+    else if (ni == 16) SS_MODE(16, MODE, grid);                                                  \
+    else SS_MODE(32, MODE, grid);                                                                \
+  } while (0)
+  if (total_chunks == 0) {
+    const dim3 grid(pblocks, heads, num_seqs);
+    SS_LAUNCH(SS_DIRECT, grid);
+    MK_LAUNCH_CHECK("ssm_scan");
+    return 0;
+  }
+  const dim3 grid(pblocks, heads, total_chunks);
+  SS_LAUNCH(SS_LOCAL, grid);
+  MK_LAUNCH_CHECK("ssm_scan (chunks)");
+  const size_t per_head = (size_t)(state_floats / heads);
+  const dim3 cgrid((unsigned)((state_floats + 255) / 256), num_seqs);
+  ssm_combine_kernel<<<cgrid, 256, 0, stream>>>(state, (size_t)slot_stride, slots, cu_q, chunk_state,
+                                                (size_t)state_floats, chunk_decay, heads, per_head);
+  MK_LAUNCH_CHECK("ssm_combine");
+  SS_LAUNCH(SS_FROM, grid);
+  MK_LAUNCH_CHECK("ssm_scan (outputs)");
 #undef SS_LAUNCH
-  MK_LAUNCH_CHECK("ssm_scan");
+#undef SS_MODE
+#undef SS_RUN
   return 0;
 }
 

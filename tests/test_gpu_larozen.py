@@ -76,7 +76,7 @@ NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "
 PORTIONS_ALONE = ((0, 21), (21, 2), (23, 9), (32, 1), (33, 1), (34, 6))
 
 
-def run_mixer_in_portions(part, x, dtype, hidden, pages=8, page=16):
+def run_mixer_in_portions(part, x, dtype, hidden, pages=8, page=16, portions=PORTIONS_ALONE):
     """The mixer over one sequence cut into PORTIONS_ALONE (pages of 16: portions end inside
     pages, two of them are single tokens), from a cache and a state slot of its own."""
     from mercury_amd.cache import CacheManager
@@ -84,7 +84,7 @@ def run_mixer_in_portions(part, x, dtype, hidden, pages=8, page=16):
     from mercury_amd.parts import LayerCache
 
     spec, state_spec = part.cache_spec(), part.state_spec()
-    part.prepare(64, DEV)
+    part.prepare(pages * page, DEV)
     from mercury_amd.parts import CacheSpec
 
     # a manager always has a cache group; a mixer without a cache leaves it unused
@@ -98,7 +98,7 @@ def run_mixer_in_portions(part, x, dtype, hidden, pages=8, page=16):
         # a slot that held something else before: the step that starts a sequence clears it
         state = torch.full((2, *state_spec.shape), 3.0, dtype=state_spec.dtype, device=DEV)
     out = []
-    for start, count in PORTIONS_ALONE:
+    for start, count in portions:
         if not manager.holds("s"):
             manager.admit("s", [], count)
         manager.grow("s", start, start + count)
@@ -192,6 +192,28 @@ def test_state_space_mixer_carries_its_state(dtype, sizes):
     got = run_mixer_in_portions(part, x, dtype, hidden)
     m = {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv, "norm_groups": parts}
     want = plain.state_space_mixer(x.float(), plain_names(params), "p.", m, 1e-5)
+    rounded = plain.state_space_mixer(x.float(), plain_names(params), "p.", m, 1e-5, plain.to_bf16)
+    close(got, want, dtype, rounded)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(64, 4, 16, 24, 2, 4, 1), (128, 2, 64, 128, 1, 3, 2)], ids=["small", "sized"])
+def test_long_portions_run_the_recurrence_in_chunks(dtype, sizes):
+    """Portions of 300, 1, 129, 128 and 2 tokens: sequences longer than a chunk of the
+    recurrence run as chunks side by side, from the state the step before left (a chunk that
+    is full to its last token, one of a single token, then direct steps again)."""
+    from mercury_amd.parts import StateSpaceMixer
+
+    hidden, heads, vdim, state, groups, conv, parts = sizes
+    part = StateSpaceMixer(hidden, heads, vdim, state, groups, conv, norm_groups=parts, eps=1e-5,
+                           names=SS_NAMES)
+    params = bind_random(part, dtype, scale=0.3, seed=19)
+    x = rnd(560, hidden, seed=34).to(dtype)
+    portions = ((0, 300), (300, 1), (301, 129), (430, 128), (558, 2))
+    got = run_mixer_in_portions(part, x, dtype, hidden, pages=40, portions=portions)
+    m = {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv, "norm_groups": parts}
+    want = plain.state_space_mixer(x.double(), {k: v.double() for k, v in plain_names(params).items()},
+                                   "p.", m, 1e-5).float()
     rounded = plain.state_space_mixer(x.float(), plain_names(params), "p.", m, 1e-5, plain.to_bf16)
     close(got, want, dtype, rounded)
 
