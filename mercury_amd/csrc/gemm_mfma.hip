@@ -850,7 +850,8 @@ extern "C" int mk_qkv_skinny_normed(const long long* h64, const void* norm_w, in
 
 // ------------------------------------------------------------------------------- tiled
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3, EPI_QKV = 4 };
+// (EPI_RELU2: EPI_BF16 with the square of relu applied to the float32 sum before it is rounded)
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3, EPI_QKV = 4, EPI_RELU2 = 5 };
 
 // a / b for 0 <= a < 2^22 and 0 < b: the float quotient is off by less than one, which one
 // step either way repairs.  A dozen instructions where the general division is forty, on
@@ -1187,7 +1188,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = acc[ta][tb][i] + col_bias[tb][i];
       const bool whole = n + 3 < N && (ldo & 3) == 0;
-      if (EPI == EPI_BF16) {
+      if (EPI == EPI_RELU2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float r = fmaxf(v[i], 0.f);
+          v[i] = r * r;
+        }
+      }
+      if (EPI == EPI_BF16 || EPI == EPI_RELU2) {
         bf16_t* dst = (bf16_t*)out_ + (size_t)m * ldo + n;
         if (whole) {
           *(uint2*)dst = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
@@ -1460,6 +1468,21 @@ extern "C" int mk_qkv_tiled(const void* x, const void* w, const void* bias, int 
   MK_REQUIRE(config < TILED_CONFIGS, "qkv projection: no configuration %d", config);
   launch_tiled<EPI_QKV>(config, x, w, bias, bias_dtype, nullptr, M, N, K, N, 1, stream, t);
   MK_LAUNCH_CHECK("qkv_tiled");
+  return 0;
+}
+
+// out = act(x W^T) as bfloat16, the activation MK_UNARY_* applied to the float32 sums in the
+// epilogue (one rounding).
+extern "C" int mk_linear_tiled_act(const void* x, const void* w, void* out, int M, int N, int K,
+                                   int act, int config, hipStream_t stream) {
+  MK_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0,
+             "tiled projection: K=%d must be a multiple of 8 (M=%d N=%d)", K, M, N);
+  MK_REQUIRE(act == MK_UNARY_RELU2, "tiled projection: unknown activation %d", act);
+  MK_REQUIRE((M + 63) / 64 <= 65535, "tiled projection: M=%d too large for one launch", M);
+  if (config < 0) config = mk_linear_tiled_config(M, N, K, 2);
+  MK_REQUIRE(config < TILED_CONFIGS, "tiled projection: no configuration %d", config);
+  launch_tiled<EPI_RELU2>(config, x, w, nullptr, MK_F32, out, M, N, K, N, 1, stream);
+  MK_LAUNCH_CHECK("linear_tiled_act");
   return 0;
 }
 

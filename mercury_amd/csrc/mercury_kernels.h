@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 28
+#define MK_ABI_VERSION 29
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
@@ -427,6 +427,11 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       int d, float scale, int window, int rows_per_tile, int staged,
                       int num_splits, int split_blocks, float* part_o, float* part_ml,
                       hipStream_t stream);
+
+// out [M, N] (bfloat16) = act(x W^T) for an activation of one operand MK_UNARY_*, applied to the
+// float32 sums in the tiled kernel's epilogue.  config -1: by the sizes.
+int mk_linear_tiled_act(const void* x, const void* w, void* out, int M, int N, int K, int act,
+                        int config, hipStream_t stream);
 
 // mk_attention_mfma in tiles of 16 rows with a say in the score: score_cap > 0 bounds the
 // scaled score to cap * tanh(score / cap); sinks (float32 [n_q], or null) adds exp(sink[head])

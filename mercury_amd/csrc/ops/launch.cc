@@ -449,6 +449,17 @@ void unary_mlp(Launch& l, const void* x, int m, int hidden, const void* w_up, co
                int inter, int act, float* h, const float*& pending, int& pending_count) {
   pending = nullptr;
   pending_count = 0;
+  // many rows on the matrix cores: the activation in the product's epilogue
+  if (mfma_eligible(l.dtype(), l.dtype(), m, hidden) && kernels().has_mfma() && !gated_is_skinny(m)) {
+    void* acted = l.alloc((size_t)m * inter * l.elem());
+    if (!l.dry()) {
+      check_mfma(need_mfma().mk_linear_tiled_act(x, w_up, acted, m, inter, hidden, act, -1,
+                                                 l.stream()), "linear_act");
+    }
+    project_into_stream(l, acted, m, w_down, hidden, inter, nullptr, kF32, h, pending,
+                        pending_count);
+    return;
+  }
   // the product in float32, so that the activation's result is rounded once
   void* up = linear(l, x, m, w_up, inter, hidden, nullptr, kF32, nullptr, kF32, false);
   void* acted = l.alloc((size_t)m * inter * l.elem());

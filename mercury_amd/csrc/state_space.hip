@@ -15,6 +15,8 @@
 // B_t, C_t, x_t, dt_t and the decay of 16 tokens at a time are staged in LDS.  The state lies
 // in memory as the lanes hold it ([head][block of 8 columns][entry][lane]), so reading and
 // writing it is contiguous: a decoded token is one read and one write of the state.
+#include <algorithm>
+
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -46,7 +48,8 @@ __global__ void causal_conv_kernel(const float* __restrict__ proj, int row_strid
   const int seq = token_seq[t];
   const int local = t - cu_q[seq];
   const float* mine = carried + (size_t)slots[seq] * slot_stride;
-  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+  // a workgroup takes 256 channels of a token: few tokens still spread over the chip
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
     float acc = weight_at<TW>(bias, c);
     for (int j = 0; j < taps; ++j) {
       const int back = taps - 1 - j;            // how many tokens before t
@@ -72,7 +75,7 @@ __global__ void conv_carry_kernel(const float* __restrict__ proj, int row_stride
   const int first = cu_q[seq], count = cu_q[seq + 1] - first;
   float* mine = carried + (size_t)slots[seq] * slot_stride;
   const int keep = taps - 1;
-  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
     // ascending k: entry k takes what entry k + count held, or this step's input
     for (int k = 0; k < keep; ++k) {
       const int at = count - keep + k;   // index among this step's tokens
@@ -299,17 +302,19 @@ extern "C" int mk_causal_conv_silu(const float* proj, int row_stride, int col0, 
   MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "causal_conv: weight dtype %d",
              weight_dtype);
   if (tokens == 0) return 0;
+  const int col_blocks = std::min(1024, (channels + 255) / 256);
+  const dim3 grid(tokens, col_blocks);
   if (weight_dtype == MK_F32)
-    causal_conv_kernel<float><<<tokens, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
+    causal_conv_kernel<float><<<grid, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
                                                            w, bias, carried, (size_t)slot_stride,
                                                            slots, token_seq, cu_q, out);
   else
-    causal_conv_kernel<bf16_t><<<tokens, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
+    causal_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
                                                             w, bias, carried, (size_t)slot_stride,
                                                             slots, token_seq, cu_q, out);
   MK_LAUNCH_CHECK("causal_conv");
   if (taps > 1) {
-    conv_carry_kernel<<<num_seqs, 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
+    conv_carry_kernel<<<dim3(num_seqs, col_blocks), 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
                                                     carried, (size_t)slot_stride, slots, cu_q);
     MK_LAUNCH_CHECK("conv_carry");
   }
