@@ -390,6 +390,11 @@ void register_builtin_ops() {
   r.add(OpKind{"embed", &run_embed, nullptr, MK_OP_FIXED_STREAM});
   r.add(OpKind{"norm", &run_norm, nullptr, MK_OP_FOLDS_PENDING | MK_OP_FIXED_STREAM});
   r.add(OpKind{"attention", &run_attention, &tiles_attention, MK_OP_READS_X | MK_OP_FIXED_STREAM});
+  // The same operations under names that are not flagged for the fixed-point stream: a norm
+  // that rounds once and an attention that norms q and k, scales its queries, takes its keys
+  // as values or has sinks keep their whole program on the float32 stream.
+  r.add(OpKind{"norm_once", &run_norm, nullptr, MK_OP_FOLDS_PENDING});
+  r.add(OpKind{"attention_prepared", &run_attention, &tiles_attention, MK_OP_READS_X});
   r.add(OpKind{"gated_mlp", &run_gated_mlp, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
   r.add(OpKind{"latent_attention", &run_latent_attention, &tiles_latent_attention, MK_OP_READS_X});
   r.add(OpKind{"routed_experts", &run_routed_experts, nullptr, MK_OP_READS_X});

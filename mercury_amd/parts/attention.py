@@ -166,7 +166,9 @@ class Attention(Mixer):
             # Reads a cache another entry fills: only the queries are projected.
             rows = self.n_q * self.head_dim
             w, b = w[:rows], None if b is None else b[:rows]
-        program.append("attention", core.attention_params(
+        # (a kind of its own where the fixed-point stream's kernels would not do the same)
+        program.append("attention_prepared" if self.prepared or self.sinks else "attention",
+                       core.attention_params(
             w_qkv=w.data_ptr(), b_qkv=ptr(b), b_qkv_dtype=bias_code(b),
             w_o=self.w_o.data_ptr(), b_o=ptr(self.b_o), b_o_dtype=bias_code(self.b_o),
             n_q=self.n_q, n_kv=self.n_kv, head_dim=self.head_dim, rotary_dim=pos.rotary_dim,

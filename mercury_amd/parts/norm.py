@@ -56,7 +56,7 @@ class RMSNorm(Norm):
 
     def lower(self, program, select_rows: bool = False) -> None:
         """`select_rows`: normalise the step's wanted rows only (before an output head)."""
-        program.append("norm", core.norm_params(
+        program.append("norm_once" if self.round_once else "norm", core.norm_params(
             self.weight.data_ptr(), ops.dtype_code(self.weight.dtype), self.eps, select_rows,
             self.round_once))
 

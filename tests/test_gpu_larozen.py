@@ -604,3 +604,71 @@ def test_command_line_and_trace_replay(tmp_path):
     torch.testing.assert_close(read(0), want[12:13], **F32)
     torch.testing.assert_close(read(1), want[[13, 19]], **F32)
     torch.testing.assert_close(read(2), want[4:5], **F32)
+
+
+# ------------------------------------------------------------------- drawn configurations
+
+
+def draw_config(seed: int) -> dict:
+    """A configuration whose every size, count, constant and the order of its layers are drawn:
+    widths that are and are not multiples of 8, one to many heads in one to as many groups,
+    head sizes the matrix cores take and others, values narrower and wider than keys, states of
+    few to many rows, convolutions over 1 to 5 tokens, loops anywhere or none."""
+    import random
+
+    from tests.larozen_cases import attention, layer, side_by_side, sink_attention, state_space
+
+    r = random.Random(seed)
+    width = r.choice([48, 64, 72, 100, 128, 136])
+    count = r.randint(1, 4)
+    layers = []
+    for _ in range(count):
+        kv = r.choice([1, 2, 3])
+        heads = kv * r.choice([1, 2, 4])
+        dim = r.choice([8, 12, 16, 32, 64])
+        if r.random() < 0.5:
+            turned = r.choice([0, 2, dim // 2, dim])
+            turned -= turned % 2
+            mixer = attention(heads, kv, dim, r.uniform(0.1, 0.5), rot=(r.uniform(50, 20000), turned) if turned else None,
+                              softcap=r.choice([None, 2.0, 15.0, 50.0]))
+            kind = "attention"
+        else:
+            vdim = r.choice([dim, 8, 24, 40])
+            groups = r.choice([1, 2, 3])
+            ss_heads = groups * r.choice([1, 2, 3])
+            ss_vdim = r.choice([4, 8, 16, 24, 40])
+            parts = r.choice([d for d in (1, 2, 3, 4, 6) if (ss_heads * ss_vdim) % d == 0])
+            mixer = side_by_side(
+                sink_attention(heads, kv, dim, vdim, r.uniform(0.1, 0.5),
+                               q_temp=(r.uniform(0.1, 1.5), r.choice([1, 3, 16, 64])) if r.random() < 0.7 else None),
+                state_space(ss_heads, ss_vdim, r.choice([4, 9, 16, 33, 64, 130]), groups, r.randint(1, 5), parts))
+            kind = "parallel"
+        layers.append(layer(kind, mixer, r.choice([0, 40, 64, 90])))
+    cfg = {"architecture": "Larozen", "vocab": r.choice([97, 256, 301]), "width": width,
+           "norm": {"eps": r.choice([1e-6, 1e-5, 1e-3])}, "layers": layers}
+    if r.random() < 0.7:
+        start = r.randint(0, count - 1)
+        cfg["loop"] = {"start": start, "stop": r.randint(start + 1, count), "times": r.randint(1, 3)}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_drawn_configurations(seed):
+    """Whole, then a portion that ends inside a page, a portion of two tokens and decoding, in
+    both dtypes, for configurations nobody chose."""
+    from mercury_amd.engine.replay import ReplaySession
+
+    cfg = draw_config(seed)
+    folder = write_folder(cfg, std=0.1, seed=100 + seed)
+    tokens = helpers.random_tokens(cfg["vocab"], 171, seed=seed)
+    want = plain.forward(cfg, plain.read_weights(folder, torch.float64), tokens).float()
+    cost = float((plain.forward(cfg, plain.read_weights(folder), tokens, plain.to_bf16) - want).abs().max())
+    for dtype in ("float32", "bfloat16"):
+        s = ReplaySession(folder, dtype, 256, max_live=2)
+        whole = s.step([entry("w", tokens)], ["w"])
+        check(whole, want, dtype, f"drawn {seed} whole {cfg}", cost)
+        rows = [s.step([entry("r", tokens[:137])], []), s.step([entry("r", tokens[137:139])], [])]
+        for i in range(139, 171):
+            rows.append(s.step([entry("r", tokens[i:i + 1])], ["r"] if i == 170 else []))
+        check(torch.cat(rows), want, dtype, f"drawn {seed} cut {cfg}", cost)
+        assert s.manager.leaked_pages() == 0
