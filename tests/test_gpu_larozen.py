@@ -116,8 +116,10 @@ def run_mixer_in_portions(part, x, dtype, hidden, pages=8, page=16, portions=POR
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sizes", [(64, 4, 2, 32, 16, 20.0), (100, 3, 1, 12, 12, 0.0),
-                                   (64, 6, 6, 16, 0, 5.0), (128, 8, 2, 64, 32, 30.0)],
-                         ids=["partly-turned", "odd-whole-turn-no-cap", "no-turn-own-kv-heads", "sized"])
+                                   (64, 6, 6, 16, 0, 5.0), (128, 8, 2, 64, 32, 30.0),
+                                   (64, 20, 1, 32, 16, 8.0)],
+                         ids=["partly-turned", "odd-whole-turn-no-cap", "no-turn-own-kv-heads", "sized",
+                              "twenty-heads-a-group"])
 def test_rotated_attention_whose_values_are_its_keys(dtype, sizes):
     from mercury_amd.parts import Attention, NoPosition, RotaryPosition
 
@@ -139,8 +141,10 @@ def test_rotated_attention_whose_values_are_its_keys(dtype, sizes):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sizes", [(64, 4, 4, 16, 24, (0.7, 8)), (100, 2, 1, 10, 10, None),
-                                   (128, 8, 2, 64, 64, (0.3, 1)), (64, 6, 3, 48, 8, (2.0, 30))],
-                         ids=["wide-values", "odd-no-temperature", "sized-every-1", "narrow-values"])
+                                   (128, 8, 2, 64, 64, (0.3, 1)), (64, 6, 3, 48, 8, (2.0, 30)),
+                                   (64, 36, 2, 32, 32, (0.4, 16))],
+                         ids=["wide-values", "odd-no-temperature", "sized-every-1", "narrow-values",
+                              "eighteen-heads-a-group"])
 def test_sink_attention(dtype, sizes):
     """Norms over the whole q and k, a temperature whose step falls inside the sequence (and
     inside a portion), sinks that take a good part of the weight, biases on all four."""
@@ -672,3 +676,66 @@ def test_drawn_configurations(seed):
             rows.append(s.step([entry("r", tokens[i:i + 1])], ["r"] if i == 170 else []))
         check(torch.cat(rows), want, dtype, f"drawn {seed} cut {cfg}", cost)
         assert s.manager.leaked_pages() == 0
+
+
+LONG = {
+    "architecture": "Larozen", "vocab": 211, "width": 128, "norm": {"eps": 1e-5},
+    "layers": [
+        {"type": "attention", "mlp": {"kind": "dense", "ff": 128},
+         "mixer": {"heads": 6, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "softcap": 12.0,
+                   "rot": {"base": 8000.0, "dims": 48}}},
+        {"type": "parallel", "mlp": None,
+         "mixer": {"left": {"heads": 4, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 0.09,
+                            "q_temp": {"coef": 0.6, "every": 256}},
+                   "right": {"heads": 2, "vdim": 32, "state": 16, "groups": 1, "conv": 3, "norm_groups": 1}}},
+    ],
+    "loop": {"start": 0, "stop": 2, "times": 2},
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_where_decoding_splits_the_keys(dtype):
+    """Head sizes the matrix cores take, a bound on the score, sinks that matter and queries
+    sharpened onto far keys, at 1,300 tokens and beyond: decoding splits every row's keys over
+    wavefronts and workgroups (the sink belongs to the first part alone), prompt portions over
+    a long prefix too, and the query temperature steps at 255, 511, 767, ... inside them."""
+    from mercury_amd.engine.replay import ReplaySession
+
+    folder = write_folder(LONG, std=0.09, seed=31, sharpen=3.0, sink=1.5)
+    w64, w32 = plain.read_weights(folder, torch.float64), plain.read_weights(folder)
+    tokens = helpers.random_tokens(LONG["vocab"], 1340, seed=9)
+    want = plain.forward(LONG, w64, tokens).float()
+    f32 = plain.forward(LONG, w32, tokens)
+    moved = tokens[:]
+    moved[:600] = helpers.random_tokens(LONG["vocab"], 600, seed=10)
+    assert (plain.forward(LONG, w32, moved)[-40:] - f32[-40:]).abs().max() > 0.02
+    cost = float((plain.forward(LONG, w32, tokens, plain.to_bf16) - want).abs().max())
+    slack = float((f32 - want).abs().max())
+
+    def compare(got, rows, what):
+        if dtype == "float32":
+            bound = F32["atol"] * max(1.0, float(want.abs().max())) + F32["rtol"] * want[rows].abs() + 1.5 * slack
+            worst = (got - want[rows]).abs()
+            assert (worst <= bound).all(), f"{what}: worst {worst.max():.3e}, plain's own {slack:.3e}"
+        else:
+            check(got, want[rows], dtype, what, cost)
+
+    s = ReplaySession(folder, dtype, 2 * 1344, page_size=16, max_live=2)
+    # whole, then decoded on
+    rows = [s.step([entry("r", tokens[:1300])], [])]
+    for i in range(1300, 1340):
+        rows.append(s.step([entry("r", tokens[i:i + 1])], ["r"] if i == 1339 else []))
+    compare(torch.cat(rows), slice(0, 1340), "whole then decoded")
+    # portions over a growing prefix beside a decoding neighbour
+    s.step([{"id": "n", "tokens": tokens[:1000], "want": []}], [])
+    got_p, got_n, at, n_at = [], [], 0, 1000
+    for count in (500, 12, 300, 2, 486):
+        out = s.step([entry("p", tokens[at:at + count]), entry("n", tokens[n_at:n_at + 1])], [])
+        got_p.append(out[:count])
+        got_n.append(out[count:])
+        at += count
+        n_at += 1
+    s.step([], ["p", "n"])
+    compare(torch.cat(got_p), slice(0, 1300), "portions over a prefix")
+    compare(torch.cat(got_n), slice(1000, 1005), "the neighbour's decoded tokens")
+    assert s.manager.leaked_pages() == 0
