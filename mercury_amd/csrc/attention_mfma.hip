@@ -652,7 +652,7 @@ __device__ __forceinline__ void staged_operands(KeyBlock<D>& blk, const uint4* l
 // maxima, sums and weighted values are combined through LDS in group order.  A long prompt's
 // last rows see thousands of keys; the groups cut that chain of dependent blocks into KG
 // shorter ones that run side by side on the same compute unit.
-template <int D, int RT, int KG>
+template <int D, int RT, int KG, bool CAP = false>
 __global__ __launch_bounds__(64 * ATTN_WAVES * KG, (RT == 1 ? (KG > 2 ? KG : 2) : 1)) void attn_staged_kernel(AttnParams p) {
   static_assert(D % 64 == 0, "256 threads bring whole 16-byte chunks of 32 keys");
   constexpr int BLOCK = 32 * D / 8;                       // 16-byte units of a block's keys (or values)
@@ -713,6 +713,8 @@ __global__ __launch_bounds__(64 * ATTN_WAVES * KG, (RT == 1 ? (KG > 2 ? KG : 2) 
   const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
   const float c = p.scale * 1.44269504088896340736f;
 
+  const float cap_in = CAP ? p.cap_in * 2.88539008177792681472f : 0.f;
+
   TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
   const int first = b0 + uniform(kgroup);                        // this group's blocks: first, first + KG, ...
   StagedRegs<D> ra = staged_fetch<D>(p, tw, first, b1, wg_kmin, wg_kmax, kvh, lane);
@@ -730,7 +732,8 @@ __global__ __launch_bounds__(64 * ATTN_WAVES * KG, (RT == 1 ? (KG > 2 ? KG : 2) 
     __syncthreads();                                                                    \
     if (((b) << 5) <= kmax && ((b) << 5) + 31 >= kmin) {                                \
       staged_operands<D>(blk, lds_k + (buf) * BLOCK, lds_v + (buf) * BLOCK, lane);      \
-      attend<D, RT, true>(st, blk, (b) << 5, c, g4, see_upto, see_from);                \
+      attend<D, RT, true, CAP>(st, blk, (b) << 5, c, g4, see_upto, see_from, cap_in,    \
+                               p.cap_out);                                              \
     }                                                                                   \
   } while (0)
   const int iterations = (b1 - b0 + KG - 1) / KG;       // the same for every group
@@ -789,6 +792,15 @@ __global__ __launch_bounds__(64 * ATTN_WAVES * KG, (RT == 1 ? (KG > 2 ? KG : 2) 
     float l = st.lsum[t];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
+    if (p.sinks) {
+      // the sink as one more key, its value zero
+      const float sink = p.sinks[head[t]] * 1.44269504088896340736f;
+      const float m_new = fmaxf(st.m[t], sink);
+      const float keep = st.m[t] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(st.m[t] - m_new);
+      l = l * keep + __builtin_amdgcn_exp2f(sink - m_new);
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) st.acc[t][dt] *= keep;
+    }
     const float inv = 1.f / l;
     bf16_t* dst = p.out + (size_t)(q0 + tok[t]) * p.out_stride + head[t] * D + g4 * 4;
 #pragma unroll
@@ -1330,6 +1342,15 @@ template <int D>
 static void launch_staged(const AttnParams& p, int rows_per_tile, int key_groups, hipStream_t stream) {
   if constexpr (D == 64 || D == 128) {   // wider heads do not fit the register file
     dim3 grid(p.num_tiles, p.n_kv);
+    if (p.cap_in != 0.f) {   // a bounded score: 16 rows a wavefront
+      if (key_groups == 1)
+        attn_staged_kernel<D, 1, 1, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
+      else if (key_groups == 2)
+        attn_staged_kernel<D, 1, 2, true><<<grid, 64 * ATTN_WAVES * 2, 0, stream>>>(p);
+      else if constexpr (D == 64)
+        attn_staged_kernel<D, 1, 4, true><<<grid, 64 * ATTN_WAVES * 4, 0, stream>>>(p);
+      return;
+    }
     if (rows_per_tile == 32)
       attn_staged_kernel<D, 2, 1><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
     else if (key_groups == 1)
@@ -1556,8 +1577,8 @@ static int attention_mfma(const void* q, int q_stride, void* out, int out_stride
                           bool merge, hipStream_t stream, float score_cap = 0.f,
                           const float* sinks = nullptr) {
   MK_REQUIRE(score_cap >= 0.f, "attention: negative score cap");
-  MK_REQUIRE((score_cap == 0.f && sinks == nullptr) || (rows_per_tile == 16 && staged == 0),
-             "attention: a bounded score or sinks run in tiles of 16 rows, keys unstaged");
+  MK_REQUIRE((score_cap == 0.f && sinks == nullptr) || (rows_per_tile == 16 && staged < 8),
+             "attention: a bounded score or sinks run in tiles of 16 rows a wavefront");
   if (int code = mk_attention_mfma_check(q_stride, out_stride, num_tiles, page_size, n_q, n_kv, d,
                                          scale, window, rows_per_tile, staged, num_splits,
                                          split_blocks, part_o && part_ml)) {
@@ -1639,12 +1660,12 @@ extern "C" int mk_attention_mfma_scored(const void* q, int q_stride, void* out, 
                                         const int* cu_q, const int* kv_len,
                                         const int* block_table, int table_stride, int page_size,
                                         int n_q, int n_kv, int d, float scale, int window,
-                                        int num_splits, int split_blocks, float score_cap,
-                                        const float* sinks, float* part_o, float* part_ml,
-                                        hipStream_t stream) {
+                                        int staged, int num_splits, int split_blocks,
+                                        float score_cap, const float* sinks, float* part_o,
+                                        float* part_ml, hipStream_t stream) {
   return attention_mfma(q, q_stride, out, out_stride, k_cache, v_cache, tile_seq, tile_row0,
                         num_tiles, cu_q, kv_len, block_table, table_stride, page_size, n_q, n_kv, d,
-                        scale, window, 16, 0, num_splits, split_blocks, part_o, part_ml, true,
+                        scale, window, 16, staged, num_splits, split_blocks, part_o, part_ml, true,
                         stream, score_cap, sinks);
 }
 

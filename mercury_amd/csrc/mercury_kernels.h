@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 29
+#define MK_ABI_VERSION 30
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
@@ -436,13 +436,14 @@ int mk_linear_tiled_act(const void* x, const void* w, void* out, int M, int N, i
 // mk_attention_mfma in tiles of 16 rows with a say in the score: score_cap > 0 bounds the
 // scaled score to cap * tanh(score / cap); sinks (float32 [n_q], or null) adds exp(sink[head])
 // once to the softmax's denominator.  tile_seq / tile_row0 null: every sequence brings one
-// token (see mk_attention_mfma).
+// token (see mk_attention_mfma).  staged: 0, or 1, 2, 4 key groups of workgroups of four
+// wavefronts that share a sequence's keys through LDS (the tile list then in steps of 64 rows).
 int mk_attention_mfma_scored(const void* q, int q_stride, void* out, int out_stride,
                              const void* k_cache, const void* v_cache, const int* tile_seq,
                              const int* tile_row0, int num_tiles, const int* cu_q,
                              const int* kv_len, const int* block_table, int table_stride,
                              int page_size, int n_q, int n_kv, int d, float scale, int window,
-                             int num_splits, int split_blocks, float score_cap,
+                             int staged, int num_splits, int split_blocks, float score_cap,
                              const float* sinks, float* part_o, float* part_ml,
                              hipStream_t stream);
 

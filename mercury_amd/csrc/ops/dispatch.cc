@@ -130,7 +130,7 @@ QkvKind choose_qkv(int x_dtype, int w_dtype, int m, int width, int k, int head_d
 AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, int n_kv, int window,
                              const std::vector<int>& counts, int max_q_len, int max_kv_len,
                              int force, int tile_rows, int staged_in, int splits_in,
-                             int split_blocks_in) {
+                             int split_blocks_in, bool scored) {
   AttentionPlan plan;
   plan.mfma = force == 2;
   if (force == 0 && dtype == kBF16) {
@@ -150,7 +150,7 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   for (int c : counts) total_rows += c;
   total_rows *= group;
   // 64-row tiles exist but run at one wavefront per SIMD; 32 rows measured fastest
-  const int max_rows = std::min(32, t.mk_attention_mfma_max_rows(head_dim));
+  const int max_rows = scored ? 16 : std::min(32, t.mk_attention_mfma_max_rows(head_dim));
   // (never wider than the rows the longest sequence brings: a decoded token's heads are one
   // tile of 16 however many sequences there are)
   while (rows < max_rows && rows < (long long)max_q_len * group &&
@@ -165,7 +165,7 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   // in workgroups of 128 rows of one sequence or of 64, the keys in one to four chains:
   // whichever instantiation the kernel library measured fastest for a step of this many
   // workgroups and blocks (`staged` 8, 16, 24; 20, 36 for the tiles of 64 rows).
-  if (staged < 0 && !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 64) {
+  if (staged < 0 && !scored && !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 64) {
     const long long wg128 = (total_rows / 128) * n_kv, wg64 = (total_rows / 64) * n_kv;
     if (wg64 < (1 << 24)) {
       const int code = t.mk_attention_mfma_wide_choice(head_dim, (int)wg128, (int)wg64, blocks,

@@ -80,10 +80,12 @@ struct AttentionPlan {
 
 // counts: tokens per sequence this step.  overrides < 0 (or 0 for splits) leave the choice
 // to the step's size.
+// `scored`: the attention bounds its score or has sinks, which the kernels of 16 rows a
+// wavefront compute (unstaged, or staged through LDS for prompts), the others not.
 AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, int n_kv, int window,
                              const std::vector<int>& counts, int max_q_len, int max_kv_len,
                              int force = 0, int tile_rows = -1, int staged = -1,
-                             int splits = 0, int split_blocks = 0);
+                             int splits = 0, int split_blocks = 0, bool scored = false);
 
 // Why the matrix-core attention would refuse to run `plan` for these sizes ("" when it takes
 // it): the kernel entry point's own argument checks, without the launch.

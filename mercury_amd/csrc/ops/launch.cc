@@ -276,15 +276,13 @@ AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
   }
   const std::vector<int> counts(step.counts, step.counts + step.num_seqs);
   if (!a.plain_scores()) {
-    // a bounded score or sinks: the matrix-core kernel of 16-row tiles, keys unstaged
-    if (force.tile_rows > 16 || force.staged > 0) {
-      throw KernelError("attention: a bounded score or sinks run in tiles of 16 rows, unstaged");
+    // a bounded score or sinks: the matrix-core kernels of 16 rows a wavefront
+    if (force.tile_rows > 16 || force.staged >= 8) {
+      throw KernelError("attention: a bounded score or sinks run in tiles of 16 rows a wavefront");
     }
-    // (decoding: the planner's own choice is 16 rows, and only then may it drop the tile list)
-    const int rows = step.max_q_len == 1 && a.n_q / a.n_kv <= 16 && force.tile_rows <= 0 ? -1 : 16;
     return plan_attention(dtype, a.head_dim, a.page_size, a.n_q, a.n_kv, a.window, counts,
-                          step.max_q_len, step.max_kv_len, force.kernel, rows, 0, force.splits,
-                          force.split_blocks);
+                          step.max_q_len, step.max_kv_len, force.kernel, force.tile_rows,
+                          force.staged, force.splits, force.split_blocks, true);
   }
   return plan_attention(dtype, a.head_dim, a.page_size, a.n_q, a.n_kv, a.window, counts,
                         step.max_q_len, step.max_kv_len, force.kernel, force.tile_rows, force.staged,
@@ -330,8 +328,8 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
                    q.q, q.stride, out, a.n_q * d, a.k_cache, a.v_cache,
                    plan.direct ? nullptr : tiles.seq, plan.direct ? nullptr : tiles.row0,
                    tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride, a.page_size, a.n_q,
-                   a.n_kv, d, a.scale, a.window, plan.splits, plan.split_blocks, a.score_cap,
-                   a.sinks, part_o, part_ml, l.stream()), "attention");
+                   a.n_kv, d, a.scale, a.window, plan.staged, plan.splits, plan.split_blocks,
+                   a.score_cap, a.sinks, part_o, part_ml, l.stream()), "attention");
     return out;
   }
   check_mfma(need_mfma().mk_attention_mfma(

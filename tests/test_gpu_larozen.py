@@ -739,3 +739,68 @@ def test_long_context_where_decoding_splits_the_keys(dtype):
     compare(torch.cat(got_p), slice(0, 1300), "portions over a prefix")
     compare(torch.cat(got_n), slice(1000, 1005), "the neighbour's decoded tokens")
     assert s.manager.leaked_pages() == 0
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("cap", [None, 6.0])
+def test_bounded_score_and_sinks_in_every_kernel_that_has_them(d, cap):
+    """Two prompts of 300 and 150 tokens, 8 heads in 2 groups: the float32-arithmetic kernel
+    in both dtypes, the matrix-core kernel of 16-row tiles unsplit and with the keys split in
+    3 and in 8 (parts that four wavefronts add up), and the kernel that stages keys through
+    LDS with 1, 2 and (heads of 64) 4 key groups, against the formula in float32."""
+    from mercury_amd.kernels import ops
+    from tests.helpers import context_from_spans
+
+    n_q, n_kv, page, lens = 8, 2, 16, [300, 150]
+    sinks = torch.linspace(-2.0, 4.0, n_q)
+    scale = d ** -0.5
+    q = [rnd(n, n_q, d, seed=50 + i, scale=1.5) for i, n in enumerate(lens)]
+    k = [rnd(n, n_kv, d, seed=60 + i, scale=1.5) for i, n in enumerate(lens)]
+    v = [rnd(n, n_kv, d, seed=70 + i) for i, n in enumerate(lens)]
+    as_bf16 = lambda t: t.to(torch.bfloat16).float()
+
+    def formula(q, k, v):
+        kk, vv = k.repeat_interleave(n_q // n_kv, 1), v.repeat_interleave(n_q // n_kv, 1)
+        score = torch.einsum("ihd,jhd->hij", q, kk) * scale
+        if cap:
+            score = cap * torch.tanh(score / cap)
+        score = score.masked_fill(~torch.ones(len(q), len(q), dtype=torch.bool).tril(), float("-inf"))
+        top = torch.maximum(score.max(-1, keepdim=True).values, sinks[:, None, None])
+        e = torch.exp(score - top)
+        p = e / (e.sum(-1, keepdim=True) + torch.exp(sinks[:, None, None] - top))
+        return torch.einsum("hij,jhd->ihd", p, vv)
+
+    per = -(-max(lens) // page)
+    table = torch.stack([torch.arange(s * per, (s + 1) * per, dtype=torch.int32) for s in range(len(lens))])
+    step = context_from_spans([(n, 0) for n in lens], DEV)
+
+    def run(dtype, **how):
+        cast = (lambda t: t) if dtype == torch.float32 else as_bf16
+        k_cache = torch.zeros(len(lens) * per, n_kv, page, d)
+        v_cache = torch.zeros_like(k_cache)
+        for s, n in enumerate(lens):
+            for pos in range(n):
+                k_cache[s * per + pos // page, :, pos % page] = k[s][pos]
+                v_cache[s * per + pos // page, :, pos % page] = v[s][pos]
+        q_flat = torch.cat([x.reshape(len(x), n_q * d) for x in q]).to(dtype).to(DEV)
+        got = ops.attention(q_flat, n_q * d, k_cache.to(dtype).to(DEV),
+                            v_cache.transpose(2, 3).contiguous().to(dtype).to(DEV), step, table.to(DEV),
+                            n_q, n_kv, d, scale, None, score_cap=cap, sinks=sinks.to(DEV), **how)
+        want = torch.cat([formula(cast(a), cast(b), cast(c)) for a, b, c in zip(q, k, v)])
+        return got.float().cpu().view(-1, n_q, d), want
+
+    got, want = run(torch.float32, kernel="generic")
+    torch.testing.assert_close(got, want, atol=2e-5, rtol=2e-5)
+    # without the sinks the result is another
+    bare = torch.cat([formula(a, b, c) for a, b, c in zip(q, k, v)])
+    variants = [dict(kernel="generic"), dict(kernel="mfma", tile_rows=16, staged=False),
+                dict(kernel="mfma", tile_rows=16, staged=False, split_override=(3, 0)),
+                dict(kernel="mfma", tile_rows=16, staged=False, split_override=(8, 0)),
+                dict(kernel="mfma", staged=1), dict(kernel="mfma", staged=2)]
+    if d == 64:
+        variants.append(dict(kernel="mfma", staged=4))
+    for how in variants:
+        got, want = run(torch.bfloat16, **how)
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2, msg=lambda m: f"{how}: {m}")
+    with pytest.raises(RuntimeError, match="16 rows a wavefront"):
+        run(torch.bfloat16, kernel="mfma", tile_rows=32)
