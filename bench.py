@@ -449,9 +449,9 @@ def larozen_configs(z: dict) -> dict:
     """name -> config.json of the two models compared at the sizes `z`."""
     scale = z["dim"] ** -0.5
     attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
-                 "scale": scale, "softcap": 30.0, "rot": {"base": 10000.0, "dims": z["dim"] // 2}}
+                 "scale": scale, "softcap": 50.0, "rot": {"base": 10000.0, "dims": z["dim"] // 2}}
     left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
-            "scale": scale, "q_temp": {"coef": 0.5, "every": 256}}
+            "scale": scale, "q_temp": {"coef": 0.4, "every": 128}}
     right = {"heads": z["ss_heads"], "vdim": z["ss_vdim"], "state": z["state"], "groups": z["groups"],
              "conv": 4, "norm_groups": z["groups"]}
     mlp = {"kind": "dense", "ff": z["ff"]}
