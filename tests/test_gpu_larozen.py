@@ -623,7 +623,7 @@ def draw_config(seed: int) -> dict:
     from tests.larozen_cases import attention, layer, side_by_side, sink_attention, state_space
 
     r = random.Random(seed)
-    width = r.choice([48, 64, 72, 100, 128, 136])
+    width = r.choice([48, 50, 64, 72, 75, 100, 128, 136])
     count = r.randint(1, 4)
     layers = []
     for _ in range(count):
@@ -656,7 +656,29 @@ def draw_config(seed: int) -> dict:
     return cfg
 
 
-@pytest.mark.parametrize("seed", range(40))
+def check_positions(got, want, rounded, what):
+    """bfloat16 on configurations that may be badly conditioned (one head, a norm over a few
+    columns): position by position.  The error of a position is the root mean square over the
+    vocabulary of the difference of the logits, their mean taken off; the engine's may be 3
+    times what rounding costs the plain implementation at that position (or at the median
+    position, where that is more); one position in fifty may be over, none by more than half."""
+    assert got.shape == want.shape and torch.isfinite(got).all(), what
+
+    def error(x):
+        d = x - want
+        return (d - d.mean(-1, keepdim=True)).pow(2).mean(-1).sqrt()
+
+    plain_cost = error(rounded)
+    allowed = 3.0 * torch.maximum(plain_cost, plain_cost.median())
+    ratio = error(got) / allowed
+    over = int((ratio > 1).sum())
+    assert ratio.max() <= 1.5 and over <= max(1, got.shape[0] // 50), (
+        f"{what}: {over} positions over, the worst {ratio.max():.2f} times its allowance "
+        f"(position {int(ratio.argmax())})")
+    assert error(got).median() <= 1.5 * plain_cost.median(), f"{what}: the median position"
+
+
+@pytest.mark.parametrize("seed", range(60))
 def test_drawn_configurations(seed):
     """Whole, then a portion that ends inside a page, a portion of two tokens and decoding, in
     both dtypes, for configurations nobody chose."""
@@ -666,15 +688,18 @@ def test_drawn_configurations(seed):
     folder = write_folder(cfg, std=0.1, seed=100 + seed)
     tokens = helpers.random_tokens(cfg["vocab"], 171, seed=seed)
     want = plain.forward(cfg, plain.read_weights(folder, torch.float64), tokens).float()
-    cost = float((plain.forward(cfg, plain.read_weights(folder), tokens, plain.to_bf16) - want).abs().max())
+    rounded = plain.forward(cfg, plain.read_weights(folder), tokens, plain.to_bf16)
     for dtype in ("float32", "bfloat16"):
         s = ReplaySession(folder, dtype, 256, max_live=2)
         whole = s.step([entry("w", tokens)], ["w"])
-        check(whole, want, dtype, f"drawn {seed} whole {cfg}", cost)
         rows = [s.step([entry("r", tokens[:137])], []), s.step([entry("r", tokens[137:139])], [])]
         for i in range(139, 171):
             rows.append(s.step([entry("r", tokens[i:i + 1])], ["r"] if i == 170 else []))
-        check(torch.cat(rows), want, dtype, f"drawn {seed} cut {cfg}", cost)
+        for got, how in ((whole, "whole"), (torch.cat(rows), "cut")):
+            if dtype == "float32":
+                check(got, want, dtype, f"drawn {seed} {how} {cfg}", 0.0)
+            else:
+                check_positions(got, want, rounded, f"drawn {seed} {how} {cfg}")
         assert s.manager.leaked_pages() == 0
 
 
