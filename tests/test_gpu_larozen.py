@@ -829,3 +829,37 @@ def test_bounded_score_and_sinks_in_every_kernel_that_has_them(d, cap):
         torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2, msg=lambda m: f"{how}: {m}")
     with pytest.raises(RuntimeError, match="16 rows a wavefront"):
         run(torch.bfloat16, kernel="mfma", tile_rows=32)
+
+
+def test_preemption_and_sampling_with_per_request_state():
+    """A pool so small that requests are preempted and start over (their state slot is given
+    back, taken again and cleared): the greedy tokens stay the plain implementation's.  Sampled
+    tokens (temperature, nucleus) do not depend on what else is in the batch."""
+    from mercury_amd import Engine, EngineConfig, SamplingParams
+
+    folder = folder_for("small")
+    cfg, weights = plain.read_config(folder), plain.read_weights(folder)
+    prompts = [helpers.random_tokens(cfg["vocab"], 60, seed=70 + i) for i in range(4)]
+
+    def greedy(prompt, count):
+        tokens = list(prompt)
+        for _ in range(count):
+            tokens.append(int(plain.forward(cfg, weights, tokens)[-1].argmax()))
+        return tokens[len(prompt):]
+
+    tight = Engine(EngineConfig(model=str(folder), device=DEV, dtype="float32", num_blocks=14,
+                                block_size=16, max_model_len=128, max_running=4,
+                                debug_invariants=True))
+    got = tight.generate(prompts, SamplingParams(ignore_eos=True), max_tokens=24)
+    assert tight.sched.stats["preemptions"] > 0
+    assert got == [greedy(p, 24) for p in prompts]
+    assert tight.leaked_blocks() == 0
+
+    def fresh():
+        return Engine(EngineConfig(model=str(folder), device=DEV, dtype="float32", num_blocks=48,
+                                   block_size=16, max_model_len=128, seed=9))
+
+    params = SamplingParams(temperature=0.9, top_p=0.8, ignore_eos=True)
+    together = fresh().generate(prompts[:3], params, max_tokens=10)
+    alone = fresh().generate(prompts[:1], params, max_tokens=10)
+    assert together[0] == alone[0] and len(set(together[0])) > 1
