@@ -863,3 +863,15 @@ def test_preemption_and_sampling_with_per_request_state():
     together = fresh().generate(prompts[:3], params, max_tokens=10)
     alone = fresh().generate(prompts[:1], params, max_tokens=10)
     assert together[0] == alone[0] and len(set(together[0])) > 1
+
+
+def test_state_layout_formula_is_the_kernel_library_s():
+    """The part sizes a request's state without the kernel library; the library says the same."""
+    from mercury_amd.hostcore import core
+    from mercury_amd.kernels import lib
+    from mercury_amd.parts import StateSpaceMixer
+
+    lib.load("core")
+    for heads, vdim, state in ((4, 16, 24), (3, 10, 9), (16, 64, 128), (2, 40, 130), (1, 33, 256), (5, 8, 4)):
+        part = StateSpaceMixer(64, heads, vdim, state, 1, 2)
+        assert part.recurrent_floats() == core.ssm_state_floats(heads, vdim, state)
