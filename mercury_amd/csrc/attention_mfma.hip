@@ -1673,6 +1673,25 @@ extern "C" int mk_attention_mfma_parts_written(int rows_per_tile, int num_splits
   return d <= 128 && attn_grouped(rows_per_tile, num_splits) ? num_splits / ATTN_WAVES : num_splits;
 }
 
+// mk_attention_mfma_parts with a bound on the score and sinks (see mk_attention_mfma_scored):
+// the part that holds the first keys carries the sink, so whoever merges the parts needs to
+// know nothing of it.
+extern "C" int mk_attention_mfma_parts_scored(const void* q, int q_stride, const void* k_cache,
+                                              const void* v_cache, const int* tile_seq,
+                                              const int* tile_row0, int num_tiles, const int* cu_q,
+                                              const int* kv_len, const int* block_table,
+                                              int table_stride, int page_size, int n_q, int n_kv,
+                                              int d, float scale, int window, int num_splits,
+                                              int split_blocks, float score_cap, const float* sinks,
+                                              float* part_o, float* part_ml, hipStream_t stream) {
+  MK_REQUIRE(num_splits > 1 && mk_attention_mfma_parts_written(16, num_splits, d) > 1,
+             "attention: partial results are left only where the keys are split over workgroups");
+  return attention_mfma(q, q_stride, nullptr, n_q * d, k_cache, v_cache, tile_seq, tile_row0,
+                        num_tiles, cu_q, kv_len, block_table, table_stride, page_size, n_q, n_kv, d,
+                        scale, window, 16, 0, num_splits, split_blocks, part_o, part_ml, false,
+                        stream, score_cap, sinks);
+}
+
 extern "C" int mk_attention_mfma_parts(const void* q, int q_stride, const void* k_cache,
                                        const void* v_cache, const int* tile_seq,
                                        const int* tile_row0, int num_tiles, const int* cu_q,

@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 30
+#define MK_ABI_VERSION 31
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
@@ -446,6 +446,15 @@ int mk_attention_mfma_scored(const void* q, int q_stride, void* out, int out_str
                              int staged, int num_splits, int split_blocks, float score_cap,
                              const float* sinks, float* part_o, float* part_ml,
                              hipStream_t stream);
+// The same, leaving the parts of split keys unmerged (see mk_attention_mfma_parts).
+int mk_attention_mfma_parts_scored(const void* q, int q_stride, const void* k_cache,
+                                   const void* v_cache, const int* tile_seq, const int* tile_row0,
+                                   int num_tiles, const int* cu_q, const int* kv_len,
+                                   const int* block_table, int table_stride, int page_size,
+                                   int n_q, int n_kv, int d, float scale, int window,
+                                   int num_splits, int split_blocks, float score_cap,
+                                   const float* sinks, float* part_o, float* part_ml,
+                                   hipStream_t stream);
 
 // Decoding with split keys, in two kernels instead of three.  mk_attention_mfma_parts is
 // mk_attention_mfma without the merge of the key splits: the partial results stay in part_o /

@@ -10,6 +10,8 @@
 //   mk_concat_cast     [a | b] row by row, in the compute dtype (the operand of a projection
 //                      of two streams);
 //   mk_copy_f32        a copy by a kernel (a captured graph records no memcpy node here).
+#include <algorithm>
+
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -20,8 +22,8 @@ __device__ __forceinline__ float weight_at(const void* w, int i) {
   return Elem<TW>::load((const TW*)w + i);
 }
 
-// One workgroup per token.  The row of qkv is [q: n_q d | k: n_kv d | v: n_kv dv], the last
-// part absent when the values are the keys.
+// One workgroup per token, or several that share its outputs.  The row of qkv is
+// [q: n_q d | k: n_kv d | v: n_kv dv], the last part absent when the values are the keys.
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const float* __restrict__ qkv, int row_stride, T* __restrict__ q_out,
@@ -77,25 +79,30 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
                     : at(base + j) * cs[j - half] + at(base + j - half) * sn[j - half];
   };
 
-  for (int i = threadIdx.x; i < qw; i += blockDim.x) {
-    const int head = i / d, j = i - head * d;
-    Elem<T>::store(q_out + (size_t)t * qw + i, turned(q_at, head * d, j));
-  }
-  if (!write_kv) return;
-
+  // The outputs [q | k | v] are dealt over the workgroups of the token (blockIdx.y): with few
+  // tokens each thread has one or two of them, and every workgroup has made the sums above
+  // for itself.
   const int page_size = 1 << page_shift;
-  const int page = block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)];
-  if (page < 0) return;  // the host never schedules a write into a page that was given back
+  const int page = write_kv ? block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)] : -1;
   const int off = pos & (page_size - 1);
-  for (int i = threadIdx.x; i < kw; i += blockDim.x) {
-    const int head = i / d, j = i - head * d;
-    const size_t dst = (((size_t)page * n_kv + head) * page_size + off) * d + j;
-    Elem<T>::store(k_cache + dst, turned(k_at, head * d, j));
-  }
+  // (the host never schedules a write into a page that was given back: page < 0 writes nothing)
+  const int vw = n_kv * dv;
+  const int total = qw + (write_kv && page >= 0 ? kw + vw : 0);
   const float* v_src = values_are_keys ? k_src : k_src + kw;
-  for (int i = threadIdx.x; i < n_kv * dv; i += blockDim.x) {
-    const int head = i / dv, j = i - head * dv;
-    Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * dv + j) * page_size + off, v_src[i]);
+  for (int idx = blockIdx.y * blockDim.x + threadIdx.x; idx < total; idx += gridDim.y * blockDim.x) {
+    if (idx < qw) {
+      const int head = idx / d, j = idx - head * d;
+      Elem<T>::store(q_out + (size_t)t * qw + idx, turned(q_at, head * d, j));
+    } else if (idx < qw + kw) {
+      const int i = idx - qw;
+      const int head = i / d, j = i - head * d;
+      const size_t dst = (((size_t)page * n_kv + head) * page_size + off) * d + j;
+      Elem<T>::store(k_cache + dst, turned(k_at, head * d, j));
+    } else {
+      const int i = idx - qw - kw;
+      const int head = i / dv, j = i - head * dv;
+      Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * dv + j) * page_size + off, v_src[i]);
+    }
   }
 }
 
@@ -206,8 +213,12 @@ extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int 
   MK_REQUIRE(!write_kv || (k_cache && v_cache && block_table), "qk_prepare: no cache to write");
   MK_REQUIRE(norm_dtype == MK_F32 || norm_dtype == MK_BF16, "qk_prepare: norm dtype %d", norm_dtype);
   if (tokens == 0) return 0;
+  // few tokens: a token's outputs over several workgroups, so that the chip is not idle
+  const int by_size = (need + 255) / 256;
+  const int chunks = std::max(1, std::min(by_size, 1024 / tokens));
+  const dim3 grid(tokens, chunks);
 #define QK_LAUNCH(T, TW)                                                                         \
-  qk_prepare_kernel<T, TW><<<tokens, 256, 0, stream>>>(                                          \
+  qk_prepare_kernel<T, TW><<<grid, 256, 0, stream>>>(                                          \
       qkv, row_stride, (T*)q_out, q_norm, k_norm, eps, temp_coef, temp_every, cos_table,         \
       sin_table, rot, interleaved, positions, token_seq, block_table, table_stride, (T*)k_cache, \
       (T*)v_cache, mk_log2(page_size), n_q, n_kv, d, dv, values_are_keys, write_kv)

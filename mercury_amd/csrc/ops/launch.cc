@@ -361,7 +361,7 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
   int heads_per_slice = 0, written = 0;
   bool wide = false;
   const bool fixed = h_fixed != nullptr || (l.dry() && l.ctx->stream_fixed);
-  if (fold != 0 && plan.mfma && a.plain_scores() && plan.splits > 1 && !plan.staged && plan.rows == 16 &&
+  if (fold != 0 && plan.mfma && plan.splits > 1 && !plan.staged && plan.rows == 16 &&
       step.max_q_len == 1 && plan.num_tiles == m && !b_o && a.n_q / a.n_kv <= 16) {
     const KernelTable& t = need_mfma();
     written = t.mk_attention_mfma_parts_written(plan.rows, plan.splits, d);
@@ -401,12 +401,21 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
   if (l.dry() || m == 0) return;
   const KernelTable& t = need_mfma();
   const mk_tile_list& tiles = tiles_for(step, a.n_q / a.n_kv, plan.tile_rows);
+  if (!a.plain_scores()) {
+    check_mfma(t.mk_attention_mfma_parts_scored(
+                   q.q, q.stride, a.k_cache, a.v_cache, plan.direct ? nullptr : tiles.seq,
+                   plan.direct ? nullptr : tiles.row0, tiles.count, s.cu_q, s.kv_len, s.table,
+                   s.table_stride, a.page_size, a.n_q, a.n_kv, d, a.scale, a.window, plan.splits,
+                   plan.split_blocks, a.score_cap, a.sinks, part_o, part_ml, l.stream()),
+               "attention");
+  } else {
   check_mfma(t.mk_attention_mfma_parts(q.q, q.stride, a.k_cache, a.v_cache,
                                        plan.direct ? nullptr : tiles.seq,
                                        plan.direct ? nullptr : tiles.row0, tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride,
                                        a.page_size, a.n_q, a.n_kv, d, a.scale, a.window, plan.rows,
                                        plan.splits, plan.split_blocks, part_o, part_ml, l.stream()),
              "attention");
+  }
   check_mfma(t.mk_attention_out(part_o, part_ml, written, w_o, out, h_fixed, m, hidden, a.n_q, a.n_kv, d,
                                 heads_per_slice, wide ? 1 : 0, l.stream()), "attention_out");
 }
