@@ -120,9 +120,9 @@ __global__ void unary_act_kernel(const TI* __restrict__ x, T* __restrict__ out, 
   Elem<T>::store(out + i, y);
 }
 
-// One workgroup per token: the two rows' sums of squares, then the weighted sum.  A thread keeps
-// its values of both rows (up to NS_KEEP each) between the two passes.
-#define NS_KEEP 8
+// A token's workgroups (blockIdx.y of them) each make the two rows' sums of squares for
+// themselves, in the same order, and then write their own share of the weighted sum: with few
+// tokens the row is spread over the chip, with many a token has one workgroup.
 template <typename TW>
 __global__ __launch_bounds__(256) void normed_sum_kernel(
     float* __restrict__ h, const float* __restrict__ ya, const float* __restrict__ pa, int na,
@@ -136,17 +136,8 @@ __global__ __launch_bounds__(256) void normed_sum_kernel(
     return v;
   };
   const bool has_b = yb != nullptr || nb > 0;
-  float va[NS_KEEP], vb[NS_KEEP];
   float sa = 0.f, sb = 0.f;
-#pragma unroll
-  for (int j = 0; j < NS_KEEP; ++j) {
-    const int i = threadIdx.x + j * blockDim.x;
-    va[j] = i < hidden ? value(ya, pa, na, i) : 0.f;
-    vb[j] = i < hidden && has_b ? value(yb, pb, nb, i) : 0.f;
-    sa += va[j] * va[j];
-    sb += vb[j] * vb[j];
-  }
-  for (int i = threadIdx.x + NS_KEEP * blockDim.x; i < hidden; i += blockDim.x) {
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     const float a = value(ya, pa, na, i);
     sa += a * a;
     if (has_b) {
@@ -156,15 +147,7 @@ __global__ __launch_bounds__(256) void normed_sum_kernel(
   }
   const float ra = rsqrtf(block_sum(sa, scratch) / (float)hidden + eps);
   const float rb = has_b ? rsqrtf(block_sum(sb, scratch) / (float)hidden + eps) : 0.f;
-#pragma unroll
-  for (int j = 0; j < NS_KEEP; ++j) {
-    const int i = threadIdx.x + j * blockDim.x;
-    if (i >= hidden) continue;
-    float sum = va[j] * ra * weight_at<TW>(wa, i);
-    if (has_b) sum += vb[j] * rb * weight_at<TW>(wb, i);
-    h[base + i] += mult * sum;
-  }
-  for (int i = threadIdx.x + NS_KEEP * blockDim.x; i < hidden; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < hidden; i += gridDim.y * blockDim.x) {
     float sum = value(ya, pa, na, i) * ra * weight_at<TW>(wa, i);
     if (has_b) sum += value(yb, pb, nb, i) * rb * weight_at<TW>(wb, i);
     h[base + i] += mult * sum;
@@ -265,11 +248,12 @@ extern "C" int mk_normed_sum(float* h, const float* ya, const float* pa, int na,
   MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "normed_sum: weight dtype %d",
              weight_dtype);
   if (tokens == 0) return 0;
+  const dim3 grid(tokens, std::max(1, std::min((hidden + 255) / 256, 512 / tokens)));
   if (weight_dtype == MK_F32)
-    normed_sum_kernel<float><<<tokens, 256, 0, stream>>>(h, ya, pa, na, wa, yb, pb, nb, wb, eps,
+    normed_sum_kernel<float><<<grid, 256, 0, stream>>>(h, ya, pa, na, wa, yb, pb, nb, wb, eps,
                                                           mult, (size_t)stride, hidden);
   else
-    normed_sum_kernel<bf16_t><<<tokens, 256, 0, stream>>>(h, ya, pa, na, wa, yb, pb, nb, wb, eps,
+    normed_sum_kernel<bf16_t><<<grid, 256, 0, stream>>>(h, ya, pa, na, wa, yb, pb, nb, wb, eps,
                                                            mult, (size_t)stride, hidden);
   MK_LAUNCH_CHECK("normed_sum");
   return 0;

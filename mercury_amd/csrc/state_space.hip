@@ -40,14 +40,17 @@ template <typename TW>
 __global__ void causal_conv_kernel(const float* __restrict__ proj, int row_stride, int col0,
                                    int channels, int taps, const void* __restrict__ w,
                                    const void* __restrict__ bias,
-                                   const float* __restrict__ carried, size_t slot_stride,
+                                   float* __restrict__ carried, size_t slot_stride,
                                    const int* __restrict__ slots,
                                    const int* __restrict__ token_seq,
                                    const int* __restrict__ cu_q, float* __restrict__ out) {
   const int t = blockIdx.x;
   const int seq = token_seq[t];
   const int local = t - cu_q[seq];
-  const float* mine = carried + (size_t)slots[seq] * slot_stride;
+  // a sequence that brings one token (decoding) also moves its carried inputs on here: the
+  // thread that read a channel's carried inputs is the only one that touches them
+  const bool single = cu_q[seq + 1] - cu_q[seq] == 1;
+  float* mine = carried + (size_t)slots[seq] * slot_stride;
   // a workgroup takes 256 channels of a token: few tokens still spread over the chip
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
     float acc = weight_at<TW>(bias, c);
@@ -63,16 +66,22 @@ __global__ void causal_conv_kernel(const float* __restrict__ proj, int row_strid
       acc = fmaf(weight_at<TW>(w, c * taps + j), u, acc);
     }
     out[(size_t)t * channels + c] = silu_f(acc);
+    if (single && taps > 1) {
+      for (int k = 0; k + 2 < taps; ++k) mine[(size_t)k * channels + c] = mine[(size_t)(k + 1) * channels + c];
+      mine[(size_t)(taps - 2) * channels + c] = proj[(size_t)t * row_stride + col0 + c];
+    }
   }
 }
 
-// After the convolution: the last taps - 1 inputs of every sequence become its carried ones.
+// After the convolution: the last taps - 1 inputs of every sequence of several tokens become
+// its carried ones.
 __global__ void conv_carry_kernel(const float* __restrict__ proj, int row_stride, int col0,
                                   int channels, int taps, float* __restrict__ carried,
                                   size_t slot_stride, const int* __restrict__ slots,
                                   const int* __restrict__ cu_q) {
   const int seq = blockIdx.x;
   const int first = cu_q[seq], count = cu_q[seq + 1] - first;
+  if (count == 1) return;     // the convolution's own kernel moved this sequence's on
   float* mine = carried + (size_t)slots[seq] * slot_stride;
   const int keep = taps - 1;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
@@ -313,7 +322,7 @@ extern "C" int mk_causal_conv_silu(const float* proj, int row_stride, int col0, 
                                                             w, bias, carried, (size_t)slot_stride,
                                                             slots, token_seq, cu_q, out);
   MK_LAUNCH_CHECK("causal_conv");
-  if (taps > 1) {
+  if (taps > 1 && tokens > num_seqs) {   // some sequence brings more than one token
     conv_carry_kernel<<<dim3(num_seqs, col_blocks), 256, 0, stream>>>(proj, row_stride, col0, channels, taps,
                                                     carried, (size_t)slot_stride, slots, cu_q);
     MK_LAUNCH_CHECK("conv_carry");
