@@ -238,12 +238,18 @@ int run_normed_sum(const void* params, mk_op_context* ctx) {
     std::snprintf(ctx->error, sizeof ctx->error, "normed_sum: %d sublayers", p.count);
     return 1;
   }
-  for (int i = 0; i < p.count; ++i) {
+  // one fill for the buffers of all sublayers (each a multiple of 64 floats apart)
+  const long long pitch = (n + 63) / 64 * 64;
+  {
+    float* all = nullptr;
     const int code = guarded(ctx, [&] {
       Launch l(ctx);
-      y[i] = zeros(l, n);
+      all = zeros(l, pitch * p.count);
     });
     if (code) return code;
+    for (int i = 0; i < p.count; ++i) y[i] = all ? all + pitch * i : nullptr;
+  }
+  for (int i = 0; i < p.count; ++i) {
     ctx->h = y[i];
     ctx->out_x = nullptr;
     ctx->out_x_rows = ctx->out_x_live = 0;
