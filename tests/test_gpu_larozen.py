@@ -875,3 +875,36 @@ def test_state_layout_formula_is_the_kernel_library_s():
     for heads, vdim, state in ((4, 16, 24), (3, 10, 9), (16, 64, 128), (2, 40, 130), (1, 33, 256), (5, 8, 4)):
         part = StateSpaceMixer(64, heads, vdim, state, 1, 2)
         assert part.recurrent_floats() == core.ssm_state_floats(heads, vdim, state)
+
+
+def test_the_benchmark_s_layer_sizes(tmp_path):
+    """The model `bench.py --larozen` times at its smaller sizes (2,048 wide, 64 state-space
+    heads of 64 columns and 128 rows, four layers, one re-entry; a smaller vocabulary), against
+    the plain implementation: whole, and 290 tokens with 40 decoded behind them."""
+    import sys
+
+    from mercury_amd.engine.replay import ReplaySession
+    from mercury_amd.weights import write_random_model
+
+    sys.path.insert(0, str(helpers.ROOT))
+    import bench
+
+    sizes = dict(bench.LAROZEN_SIZES["small"], vocab=2000)
+    cfg = bench.larozen_configs(sizes)["larozen"]
+    folder = write_random_model(tmp_path / "m", cfg, seed=3, std=0.02, dtype=torch.bfloat16)
+    tokens = helpers.random_tokens(cfg["vocab"], 330, seed=1)
+    weights = plain.read_weights(folder)
+    want = plain.forward(cfg, {k: v.double() for k, v in weights.items()}, tokens).float()
+    rounded = plain.forward(cfg, weights, tokens, plain.to_bf16)
+    for dtype in ("float32", "bfloat16"):
+        s = ReplaySession(folder, dtype, 512, max_live=2)
+        whole = s.step([entry("w", tokens)], ["w"])
+        rows = [s.step([entry("r", tokens[:290])], [])]
+        for i in range(290, 330):
+            rows.append(s.step([entry("r", tokens[i:i + 1])], ["r"] if i == 329 else []))
+        for got, how in ((whole, "whole"), (torch.cat(rows), "cut")):
+            if dtype == "float32":
+                check(got, want, dtype, f"benchmark sizes {how}", 0.0)
+            else:
+                check_positions(got, want, rounded, f"benchmark sizes {how}")
+        assert s.manager.leaked_pages() == 0
