@@ -112,7 +112,10 @@ __device__ __forceinline__ int chunks_of(int tokens) { return (tokens + SS_CHUNK
 // lane -> (column within the wavefront's 8, slice of n); entry i of a lane is
 // n = (i / 4) * 32 + slice * 4 + i % 4, so that four entries are one 16-byte LDS read and the
 // eight slices read 128 contiguous bytes.
-template <int NI, typename TW, int MODE>
+// CPL: columns a lane holds (1 or 2).  With two, a wavefront owns 16 columns (two blocks of 8
+// side by side in the state's layout) and reads B and C once for both: the LDS pipe, which the
+// four SIMDs of a compute unit share, is what this loop waits for first.
+template <int NI, typename TW, int MODE, int CPL>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(
     const float* __restrict__ xbc, int xbc_stride, const float* __restrict__ proj,
     int proj_stride, int z_col, int dt_col, const void* __restrict__ dt_bias,
@@ -123,8 +126,9 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
   constexpr int NPAD = NI * 8;
   __shared__ __attribute__((aligned(16))) float sB[SS_TOKENS][NPAD];
   __shared__ __attribute__((aligned(16))) float sC[SS_TOKENS][NPAD];
-  __shared__ float sX[SS_TOKENS][SS_COLS];
-  __shared__ float sZ[SS_TOKENS][SS_COLS];
+  constexpr int COLS = SS_COLS * CPL;                   // columns of the workgroup
+  __shared__ float sX[SS_TOKENS][COLS];
+  __shared__ float sZ[SS_TOKENS][COLS];
   __shared__ float sDt[SS_TOKENS], sDecay[SS_TOKENS];
 
   const int head = blockIdx.y, pblock = blockIdx.x;
@@ -145,18 +149,24 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
   }
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int slice = lane >> 3, col_in_wave = lane & 7;
-  const int col = pblock * SS_COLS + wave * 8 + col_in_wave;   // column p of the head
+  // column c of the lane is column (wave * CPL + c) * 8 + col_in_wave of the workgroup
+  const int wave_col0 = pblock * COLS + wave * CPL * 8;
   const int group = head / (heads / groups);
   const int inner = heads * P;
-  const int blocks8 = (P + SS_COLS - 1) / SS_COLS * (SS_COLS / 8);   // whole workgroups
+  const int blocks8 = (P + SS_COLS - 1) / SS_COLS * (SS_COLS / 8);   // whole workgroups of 32
 
-  const size_t within = ((size_t)head * blocks8 + (size_t)pblock * 4 + wave) * NI * 64;
+  const size_t within = ((size_t)head * blocks8 + (size_t)(pblock * 4 + wave) * CPL) * NI * 64;
   float* mine = MODE == SS_DIRECT ? state + (size_t)slots[seq] * slot_stride + within
                                   : chunk_state + (size_t)blockIdx.z * chunk_stride + within;
-  const bool live = pblock * SS_COLS + wave * 8 < P;    // the wavefront has columns at all
-  float S[NI];
+  bool live[CPL];                                       // the block of 8 has columns at all
+  float S[CPL][NI];
 #pragma unroll
-  for (int i = 0; i < NI; ++i) S[i] = (MODE != SS_LOCAL && live) ? mine[i * 64 + lane] : 0.f;
+  for (int c = 0; c < CPL; ++c) {
+    live[c] = wave_col0 + c * 8 < P;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      S[c][i] = (MODE != SS_LOCAL && live[c]) ? mine[((size_t)c * NI + i) * 64 + lane] : 0.f;
+  }
 
   const float rate = expf(weight_at<TW>(a_log, head));
   const float bias = weight_at<TW>(dt_bias, head);
@@ -172,9 +182,9 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
       sB[tt][n] = n < N ? row[group * N + n] : 0.f;
       if (MODE != SS_LOCAL) sC[tt][n] = n < N ? row[groups * N + group * N + n] : 0.f;
     }
-    for (int idx = tid; idx < n_tok * SS_COLS; idx += 256) {
-      const int tt = idx / SS_COLS, c = idx - tt * SS_COLS;
-      const int p = pblock * SS_COLS + c;
+    for (int idx = tid; idx < n_tok * COLS; idx += 256) {
+      const int tt = idx / COLS, c = idx - tt * COLS;
+      const int p = pblock * COLS + c;
       const size_t tok = first + t0 + tt;
       sX[tt][c] = p < P ? xbc[tok * xbc_stride + head * P + p] : 0.f;
       if (MODE != SS_LOCAL) sZ[tt][c] = p < P ? proj[tok * proj_stride + z_col + head * P + p] : 0.f;
@@ -188,50 +198,72 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
     }
     __syncthreads();
     for (int tt = 0; tt < n_tok; ++tt) {
-      const float x = sX[tt][wave * 8 + col_in_wave];
-      const float dtx = sDt[tt] * x, decay = sDecay[tt];
+      const float decay = sDecay[tt];
+      float x[CPL], dtx[CPL];
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        x[c] = sX[tt][(wave * CPL + c) * 8 + col_in_wave];
+        dtx[c] = sDt[tt] * x[c];
+      }
       if (MODE == SS_LOCAL) {
         dt_sum += sDt[tt];
 #pragma unroll
         for (int i4 = 0; i4 < NI / 4; ++i4) {
           const float4 b = *(const float4*)&sB[tt][i4 * 32 + slice * 4];
-          float* s = &S[i4 * 4];
-          s[0] = fmaf(decay, s[0], dtx * b.x);
-          s[1] = fmaf(decay, s[1], dtx * b.y);
-          s[2] = fmaf(decay, s[2], dtx * b.z);
-          s[3] = fmaf(decay, s[3], dtx * b.w);
+#pragma unroll
+          for (int c = 0; c < CPL; ++c) {
+            float* s = &S[c][i4 * 4];
+            s[0] = fmaf(decay, s[0], dtx[c] * b.x);
+            s[1] = fmaf(decay, s[1], dtx[c] * b.y);
+            s[2] = fmaf(decay, s[2], dtx[c] * b.z);
+            s[3] = fmaf(decay, s[3], dtx[c] * b.w);
+          }
         }
         continue;
       }
-      // four sums side by side (entries i % 4), added up at the end: ((y0 + y1) + (y2 + y3))
-      float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
+      // per column four sums side by side (entries i % 4), added up at the end:
+      // ((y0 + y1) + (y2 + y3))
+      float y0[CPL], y1[CPL], y2[CPL], y3[CPL];
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) y0[c] = y1[c] = y2[c] = y3[c] = 0.f;
 #pragma unroll
       for (int i4 = 0; i4 < NI / 4; ++i4) {
         const float4 b = *(const float4*)&sB[tt][i4 * 32 + slice * 4];
-        const float4 c = *(const float4*)&sC[tt][i4 * 32 + slice * 4];
-        float* s = &S[i4 * 4];
-        s[0] = fmaf(decay, s[0], dtx * b.x);
-        s[1] = fmaf(decay, s[1], dtx * b.y);
-        s[2] = fmaf(decay, s[2], dtx * b.z);
-        s[3] = fmaf(decay, s[3], dtx * b.w);
-        y0 = fmaf(s[0], c.x, y0);
-        y1 = fmaf(s[1], c.y, y1);
-        y2 = fmaf(s[2], c.z, y2);
-        y3 = fmaf(s[3], c.w, y3);
+        const float4 cc = *(const float4*)&sC[tt][i4 * 32 + slice * 4];
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+          float* s = &S[c][i4 * 4];
+          s[0] = fmaf(decay, s[0], dtx[c] * b.x);
+          s[1] = fmaf(decay, s[1], dtx[c] * b.y);
+          s[2] = fmaf(decay, s[2], dtx[c] * b.z);
+          s[3] = fmaf(decay, s[3], dtx[c] * b.w);
+          y0[c] = fmaf(s[0], cc.x, y0[c]);
+          y1[c] = fmaf(s[1], cc.y, y1[c]);
+          y2[c] = fmaf(s[2], cc.z, y2[c]);
+          y3[c] = fmaf(s[3], cc.w, y3[c]);
+        }
       }
-      float y = (y0 + y1) + (y2 + y3);
-      y += __shfl_xor(y, 8, MK_WAVE);
-      y += __shfl_xor(y, 16, MK_WAVE);
-      y += __shfl_xor(y, 32, MK_WAVE);
-      if (slice == 0 && col < P) {
-        const float z = sZ[tt][wave * 8 + col_in_wave];
-        y_out[(size_t)(first + t0 + tt) * inner + head * P + col] = (y + skip * x) * silu_f(z);
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        float y = (y0[c] + y1[c]) + (y2[c] + y3[c]);
+        y += __shfl_xor(y, 8, MK_WAVE);
+        y += __shfl_xor(y, 16, MK_WAVE);
+        y += __shfl_xor(y, 32, MK_WAVE);
+        const int col = wave_col0 + c * 8 + col_in_wave;   // column p of the head
+        if (slice == 0 && col < P) {
+          const float z = sZ[tt][(wave * CPL + c) * 8 + col_in_wave];
+          y_out[(size_t)(first + t0 + tt) * inner + head * P + col] = (y + skip * x[c]) * silu_f(z);
+        }
       }
     }
   }
-  if (MODE != SS_FROM && live) {
+  if (MODE != SS_FROM) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) mine[i * 64 + lane] = S[i];
+    for (int c = 0; c < CPL; ++c) {
+      if (!live[c]) continue;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) mine[((size_t)c * NI + i) * 64 + lane] = S[c][i];
+    }
   }
   if (MODE == SS_LOCAL && pblock == 0 && tid == 0) {
     chunk_decay[(size_t)blockIdx.z * heads + head] = expf(-rate * dt_sum);
@@ -366,12 +398,22 @@ extern "C" int mk_ssm_scan(const float* xbc, int xbc_stride, const float* proj, 
   MK_REQUIRE(total_chunks != 0 || (long long)num_seqs * SS_CHUNK >= tokens,
              "ssm_scan: a sequence longer than a chunk runs in chunks");
   if (tokens == 0 || num_seqs == 0) return 0;
-  const int pblocks = (P + SS_COLS - 1) / SS_COLS;
+  // Two columns a lane where the head's workgroups of 32 columns come in pairs (the layout of
+  // the state is the same either way) and a lane's registers hold twice the entries.
+  const int blocks32 = (P + SS_COLS - 1) / SS_COLS;
   const int ni = entries_for(N);
+  const int cpl = (blocks32 % 2 == 0 && ni <= 16) ? 2 : 1;
+  const int pblocks = blocks32 / cpl;
   float* chunk_state = workspace;
   float* chunk_decay = workspace ? workspace + (size_t)total_chunks * state_floats : nullptr;
 #define SS_RUN(NI, TW, MODE, grid)                                                              \
-  ssm_scan_kernel<NI, TW, MODE><<<grid, 256, 0, stream>>>(                                       \
+  if (cpl == 2)                                                                                 \
+    ssm_scan_kernel<NI, TW, MODE, 2><<<grid, 256, 0, stream>>>(                                  \
+        xbc, xbc_stride, proj, proj_stride, z_col, dt_col, dt_bias, a_log, d_skip, state,       \
+        (size_t)slot_stride, slots, cu_q, heads, P, N, groups, y_out, chunk_state,              \
+        (size_t)state_floats, chunk_decay);                                                     \
+  else                                                                                          \
+  ssm_scan_kernel<NI, TW, MODE, 1><<<grid, 256, 0, stream>>>(                                    \
       xbc, xbc_stride, proj, proj_stride, z_col, dt_col, dt_bias, a_log, d_skip, state,         \
       (size_t)slot_stride, slots, cu_q, heads, P, N, groups, y_out, chunk_state,                \
       (size_t)state_floats, chunk_decay)
